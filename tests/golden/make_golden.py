@@ -1,0 +1,80 @@
+"""Writes tests/golden/ref_vectors.npz from the reference's own C code
+compiled in place (oracle/_ref, built by `make -C oracle ref`). Run in the
+container that holds the reference tree:
+
+    python tests/golden/make_golden.py
+
+The file holds inputs' seeds/shapes and the reference's outputs only (data,
+no reference text). Tables, ids and RNG draws come from the IEEE build of the
+reference sources (bit-exact targets); attention / norm / rope outputs come
+from the build with the reference Makefile's flags (tolerance targets).
+"""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+
+import oracle  # noqa: E402
+import refcalls as R  # noqa: E402
+
+
+def inputs(seed, *shape):
+    """Deterministic inputs shared with the test: numpy PCG64 normal draws."""
+    return np.random.default_rng(seed).standard_normal(shape).astype(np.float32)
+
+
+def main():
+    ref, refi = oracle.reference(), oracle.reference(ieee=True)
+    assert ref is not None and refi is not None, "build oracle/_ref first"
+    g = {}
+    # --- seeded inputs
+    for seed in (0, 1, 42):
+        g[f"rng_uniform_{seed}"] = R.rng_u64(refi, seed, 32)
+        g[f"rng_normal_{seed}"] = R.randn(refi, seed, 256)
+    # --- tables (bit-exact targets)
+    g["flux2_cos"], g["flux2_sin"] = R.flux2_joint_compact(refi, 8, 4, 5, [(2, 3), (3, 2)])
+    g["flux3_cos"], g["flux3_sin"] = R.flux3_joint_rope(refi, 8, 4, 5, [(2, 3), (3, 2)])
+    g["qwen3_cos"], g["qwen3_sin"] = R.qwen3_rope_table(refi, 24, 128, 1e6)
+    mask = np.r_[np.ones(15), np.zeros(9)].astype(np.int32)
+    g["qwen3_f3_cos"], g["qwen3_f3_sin"] = R.qwen3_rope_table(refi, 24, 128, 1e6, mask=mask, flux3_mode=True)
+    for ax, (d, n) in enumerate(((32, 40), (48, 40), (48, 40))):
+        g[f"zimage_cos_{ax}"], g[f"zimage_sin_{ax}"] = R.zi_axis_table(refi, ax, (32, 48, 48), (n, n, n))
+    g["rope_freqs"] = R.rope_freqs(refi, [0, 1, 7, 300], 128, 10000.0)
+    # --- f32 operators (tolerance targets)
+    x = inputs(100, 6, 3, 128)
+    w = (1 + 0.02 * inputs(101, 128)).astype(np.float32)
+    g["head_rms_norm"] = R.flux3_head_rms_norm(ref, x, w, 1e-6)
+    g["rope_pairs"] = R.flux3_apply_rope(ref, x[:6], g["flux2_cos"][8:14], g["flux2_sin"][8:14])
+    q4 = x[None]
+    fr = R.rope_freqs(refi, np.arange(6), 128, 1e6)
+    g["rope_split"] = R.apply_rope_interleaved(ref, q4, fr)[0]
+    g["softmax"] = R.softmax_rows(ref, inputs(102, 5, 37) * 4)
+    for name, (sq, sk) in {"small": (5, 9), "edge": (64, 128), "tiled": (65, 129)}.items():
+        Q, K, V = inputs(110, sq, 64), inputs(111, sk, 64), inputs(112, sk, 64)
+        g[f"flash_{name}"] = R.attention_flash(ref, Q, K, V, 2, 1 / np.sqrt(32))
+    # Z-Image masked chain and Qwen3 causal GQA chain (see test for the inputs)
+    orc = oracle.oracle()
+    dims = (8, 12, 12)
+    pos, zmask, ip, cp = orc.zimage_positions(img_seq=27, wt=9, cap_seq=5)
+    seq, dim = ip + cp, 64
+    g["zi_attention"] = R.zi_attention(ref, inputs(120, seq, dim), inputs(121, dim, dim) / 8, inputs(122, dim, dim) / 8,
+                                       inputs(123, dim, dim) / 8, np.eye(dim, dtype=np.float32),
+                                       1 + 0.02 * inputs(124, 32), 1 + 0.02 * inputs(125, 32), pos, zmask, 2, dims)
+    g["zi_pos"], g["zi_mask"] = pos, zmask
+    heads, kv, hd, hidden, seq = 8, 2, 32, 24, 40
+    qmask = np.r_[np.ones(23), np.zeros(17)].astype(np.int32)
+    attn, rq, rk, rv = R.qwen3_attention(ref, inputs(130, seq, hidden), inputs(131, heads * hd, hidden) / 5,
+                                         inputs(132, kv * hd, hidden) / 5, inputs(133, kv * hd, hidden) / 5,
+                                         1 + 0.02 * inputs(134, hd), 1 + 0.02 * inputs(135, hd), qmask, heads, kv, hd)
+    g["qwen3_attention"], g["qwen3_q"], g["qwen3_k"] = attn, rq, rk
+    out = os.path.join(HERE, "ref_vectors.npz")
+    np.savez_compressed(out, **g)
+    print("wrote", out, os.path.getsize(out), "bytes,", len(g), "arrays")
+
+
+if __name__ == "__main__":
+    main()

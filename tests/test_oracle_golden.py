@@ -1,0 +1,104 @@
+"""Oracle against the committed golden vectors (tests/golden/ref_vectors.npz,
+written by tests/golden/make_golden.py from the reference's own compiled
+code). Runs anywhere: needs neither the reference tree nor a GPU.
+"""
+import os
+
+import numpy as np
+import pytest
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_vectors.npz")
+
+
+@pytest.fixture(scope="module")
+def gold():
+    return np.load(GOLD, allow_pickle=False)
+
+
+def inputs(seed, *shape):
+    return np.random.default_rng(seed).standard_normal(shape).astype(np.float32)
+
+
+def same_bits(a, b):
+    a = np.ascontiguousarray(a, dtype=np.float32); b = np.ascontiguousarray(b, dtype=np.float32)
+    return a.shape == b.shape and np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+@pytest.mark.parametrize("seed", [0, 1, 42])
+def test_rng_bit_exact(orc, gold, seed):
+    st = orc.rng(seed)
+    assert same_bits(np.array([orc.rng_uniform(st) for _ in range(32)], np.float32), gold[f"rng_uniform_{seed}"])
+    assert same_bits(orc.randn(orc.rng(seed), 256), gold[f"rng_normal_{seed}"])
+
+
+def test_tables_bit_exact(orc, gold):
+    c, s = orc.flux2_joint_tables(8, 4, 5, [(2, 3), (3, 2)])
+    assert same_bits(c, gold["flux2_cos"]) and same_bits(s, gold["flux2_sin"])
+    c, s = orc.flux3_rope_rows(orc.flux3_joint_positions(8, 4, 5, [(2, 3), (3, 2)]))
+    assert same_bits(c, gold["flux3_cos"]) and same_bits(s, gold["flux3_sin"])
+    c, s = orc.qwen3_rope_table(24, 128, 1e6)
+    assert same_bits(c, gold["qwen3_cos"]) and same_bits(s, gold["qwen3_sin"])
+    mask = np.r_[np.ones(15), np.zeros(9)].astype(np.int32)
+    c, s = orc.qwen3_rope_table(24, 128, 1e6, mask=mask, pad_at_one=True)
+    assert same_bits(c, gold["qwen3_f3_cos"]) and same_bits(s, gold["qwen3_f3_sin"])
+    for ax, d in enumerate((32, 48, 48)):
+        c, s = orc.zimage_axis_table(d, 40)
+        assert same_bits(c, gold[f"zimage_cos_{ax}"]) and same_bits(s, gold[f"zimage_sin_{ax}"])
+    assert same_bits(orc.rope_freqs_interleaved([0, 1, 7, 300], 128, 10000.0), gold["rope_freqs"])
+
+
+def test_zimage_ids_bit_exact(orc, gold):
+    pos, mask, ip, cp = orc.zimage_positions(img_seq=27, wt=9, cap_seq=5)
+    assert np.array_equal(pos, gold["zi_pos"]) and np.array_equal(mask, gold["zi_mask"])
+
+
+def test_elementwise_ops(orc, gold):
+    x = inputs(100, 6, 3, 128)
+    w = (1 + 0.02 * inputs(101, 128)).astype(np.float32)
+    np.testing.assert_allclose(orc.rms_norm_rows(x.reshape(18, 128), w, 1e-6).reshape(6, 3, 128), gold["head_rms_norm"], rtol=1e-5)
+    np.testing.assert_allclose(orc.rope_pairs(x, gold["flux2_cos"][8:14], gold["flux2_sin"][8:14]), gold["rope_pairs"], rtol=2e-6, atol=1e-7)
+    c, s = orc.qwen3_rope_table(6, 128, 1e6)
+    np.testing.assert_allclose(orc.rope_split(x, c, s), gold["rope_split"], rtol=2e-6, atol=1e-7)
+    np.testing.assert_allclose(orc.softmax_rows(inputs(102, 5, 37) * 4), gold["softmax"], rtol=2e-6, atol=1e-9)
+
+
+@pytest.mark.parametrize("name,sq,sk", [("small", 5, 9), ("edge", 64, 128), ("tiled", 65, 129)])
+def test_flash_attention(orc, gold, name, sq, sk):
+    Q, K, V = inputs(110, sq, 64), inputs(111, sk, 64), inputs(112, sk, 64)
+    np.testing.assert_allclose(orc.attention_flash(Q, K, V, 2, 1 / np.sqrt(32)), gold[f"flash_{name}"], rtol=2e-5, atol=2e-6)
+    np.testing.assert_allclose(orc.attention_strided(Q, K, V, 2, 2, 1 / np.sqrt(32)), gold[f"flash_{name}"], rtol=1e-4, atol=1e-5)
+
+
+def test_zimage_masked_chain(orc, gold):
+    dims, heads, hd, dim = (8, 12, 12), 2, 32, 64
+    pos, mask = gold["zi_pos"], gold["zi_mask"]
+    seq = pos.shape[0]
+    x = inputs(120, seq, dim).astype(np.float64)
+    wq, wk, wv = (inputs(s, dim, dim) / 8 for s in (121, 122, 123))
+    nq, nk = 1 + 0.02 * inputs(124, 32), 1 + 0.02 * inputs(125, 32)
+    q = (x @ wq.T.astype(np.float64)).astype(np.float32).reshape(seq, heads, hd)
+    k = (x @ wk.T.astype(np.float64)).astype(np.float32).reshape(seq, heads, hd)
+    v = (x @ wv.T.astype(np.float64)).astype(np.float32)
+    c, s = orc.zimage_gather(pos, axes_dims=dims)
+    q = orc.head_norm_rope_f32(q, nq, c, s, 1e-5, 0).reshape(seq, dim)
+    k = orc.head_norm_rope_f32(k, nk, c, s, 1e-5, 0).reshape(seq, dim)
+    got = orc.attention_strided(q, k, v, heads, heads, 1 / np.sqrt(hd), key_mask=mask)
+    np.testing.assert_allclose(got, gold["zi_attention"], rtol=2e-4, atol=2e-5)
+
+
+def test_qwen3_causal_gqa_chain(orc, gold):
+    heads, kv, hd, hidden, seq = 8, 2, 32, 24, 40
+    mask = np.r_[np.ones(23), np.zeros(17)].astype(np.int32)
+    x = inputs(130, seq, hidden).astype(np.float64)
+    wq, wk, wv = inputs(131, heads * hd, hidden) / 5, inputs(132, kv * hd, hidden) / 5, inputs(133, kv * hd, hidden) / 5
+    nq, nk = 1 + 0.02 * inputs(134, hd), 1 + 0.02 * inputs(135, hd)
+    q = (x @ wq.T.astype(np.float64)).astype(np.float32).reshape(seq, heads, hd)
+    k = (x @ wk.T.astype(np.float64)).astype(np.float32).reshape(seq, kv, hd)
+    v = (x @ wv.T.astype(np.float64)).astype(np.float32)
+    c, s = orc.qwen3_rope_table(seq, hd, 1e6)
+    q = orc.head_norm_rope_f32(q, nq, c, s, 1e-6, 1).reshape(seq, -1)
+    k = orc.head_norm_rope_f32(k, nk, c, s, 1e-6, 1).reshape(seq, -1)
+    np.testing.assert_allclose(q, gold["qwen3_q"], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(k, gold["qwen3_k"], rtol=1e-4, atol=1e-5)
+    got = orc.attention_strided(q, k, v, heads, kv, 1 / np.sqrt(hd), causal=True, key_mask=mask)
+    np.testing.assert_allclose(got, gold["qwen3_attention"], rtol=2e-4, atol=2e-5)
