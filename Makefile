@@ -1,0 +1,44 @@
+# MI355X (gfx950) backend of the iris attention hot path.
+#
+#   make rocm     -> iris_c_amd/libiris_dev.so   (host C + HIP kernels, C ABI of include/iris_dev.h)
+#   make oracle   -> oracle/*.so                  (CPU checker; test infrastructure)
+#   make test-cpu / test-gpu / bench
+ROCM_HOME ?= /opt/rocm
+HIPCC     ?= $(ROCM_HOME)/bin/hipcc
+CC        ?= gcc
+GPU_ARCH  ?= gfx950
+
+CSRC   = iris_c_amd/csrc
+OUT    = iris_c_amd/libiris_dev.so
+# Packed-f32 instruction selection is switched off for all device code.
+HIPFLAGS = -O3 --offload-arch=$(GPU_ARCH) -fPIC -std=c++17 -Xclang -target-feature -Xclang -packed-fp32-ops \
+           -I$(CSRC) -Iinclude
+CFLAGS   = -O2 -fPIC -Wall -Wextra -std=c11 -I$(CSRC) -Iinclude -I$(ROCM_HOME)/include
+
+HIP_SRCS = $(CSRC)/qknorm_rope.hip $(CSRC)/fa_fwd_gfx950.hip $(CSRC)/attn_generic.hip
+HIP_OBJS = $(HIP_SRCS:.hip=.o)
+
+.PHONY: rocm oracle clean test-cpu test-gpu bench
+rocm: $(OUT)
+
+$(CSRC)/%.o: $(CSRC)/%.hip $(CSRC)/iris_kernels_hip.h
+	$(HIPCC) $(HIPFLAGS) -c $< -o $@
+
+$(CSRC)/iris_rocm.o: $(CSRC)/iris_rocm.c include/iris_dev.h $(CSRC)/iris_kernels_hip.h
+	$(CC) $(CFLAGS) -c $< -o $@
+
+$(OUT): $(HIP_OBJS) $(CSRC)/iris_rocm.o
+	$(HIPCC) --offload-arch=$(GPU_ARCH) -shared -o $@ $^ -L$(ROCM_HOME)/lib -lamdhip64
+
+oracle:
+	$(MAKE) -C oracle all
+
+test-cpu:
+	python -m pytest tests -x -q -m "not gpu"
+test-gpu:
+	python -u -m pytest tests -x -v -m gpu --timeout 120 --timeout-method thread
+bench:
+	python bench.py
+
+clean:
+	rm -f $(CSRC)/*.o $(OUT)

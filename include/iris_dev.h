@@ -1,0 +1,100 @@
+/*
+ * Device (GPU) compute API of the attention hot path, MI355X (gfx950) backend.
+ *
+ * This is the C ABI of libiris_dev.so. Every declaration below that cites
+ * the reference header keeps that header's name, argument order, units and
+ * meaning, so host C code written against the reference's iris_dev.h
+ * (FLUX.2 / FLUX.3 / Z-Image transformers, Qwen3 encoder) links against
+ * this library for these calls without change.
+ *
+ * Conventions (reference iris_dev.h:7-15):
+ *  - tensors are plain device pointers from iris_dev_alloc(); bf16 values are
+ *    stored as uint16_t; matrices are row-major; strides count elements;
+ *  - operations are enqueued in order on one stream owned by the library;
+ *    results are visible to later operations, and to the host after
+ *    iris_dev_download() or iris_dev_sync();
+ *  - compute entries return void: on failure a line prefixed "iris_dev:"
+ *    goes to stderr, the output is left undefined and the process goes on
+ *    (reference iris_cuda.cu:108-111). There is no CPU fallback here.
+ *  - one caller thread, device 0.
+ */
+#ifndef IRIS_DEV_H
+#define IRIS_DEV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- setup (reference iris_dev.h:27-31, iris_cuda.cu:117-173) ---- */
+int iris_dev_init(void);            /* 1 if a usable gfx950 GPU was found */
+int iris_dev_available(void);
+const char *iris_dev_name(void);
+void iris_dev_cleanup(void);
+
+/* ---- memory (reference iris_dev.h:33-43, iris_cuda.cu:175-230) ---- */
+void *iris_dev_alloc(size_t bytes);                 /* NULL on failure; 0 bytes allocates 1 */
+void iris_dev_free(void *p);                        /* waits for pending work first */
+void iris_dev_upload(void *dst, const void *src, size_t bytes);     /* returns after the copy */
+void iris_dev_download(void *dst, const void *src, size_t bytes);   /* returns after the copy */
+void iris_dev_upload_2d(void *dst, size_t dst_stride, const void *src, size_t src_stride,
+                        size_t row_bytes, size_t rows);             /* strides in bytes */
+void iris_dev_sync(void);
+
+/* ---- the hot path ---- */
+
+/* reference iris_dev.h:74-81 (kernel iris_cuda.cu:402-420, launcher :445-453).
+ * In place on the bf16 heads x[s, h * head_dim + d] (row stride ld): per-head
+ * RMSNorm with weight w [head_dim], then rotation by the angles of row s
+ * (rope_cos/sin: [seq, head_dim / 2]). Pairs are consecutive (2i, 2i + 1),
+ * or (i, i + head_dim / 2) when split_half is set. */
+void iris_dev_head_norm_rope(uint16_t *x, int ld, const float *w,
+                             const float *rope_cos, const float *rope_sin,
+                             int seq, int heads, int head_dim, float eps,
+                             int split_half);
+
+/* reference iris_dev.h:83-92 (dispatcher iris_cuda.cu:878-937).
+ * Scaled dot-product attention over bf16 [seq, heads * head_dim] tensors.
+ * q, k, v share the row stride ldi, out has row stride ldo. With fewer kv
+ * heads (GQA), query head h uses kv head h / (heads / kv_heads).
+ * causal: query i ignores keys j > i. key_mask: device int [seq_k],
+ * 0 = ignored key, or NULL. A query with no valid key gives a zero row
+ * (reference iris_cuda.cu:531, 650, 676). */
+void iris_dev_attention(uint16_t *out, int ldo,
+                        const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                        int ldi, int seq_q, int seq_k, int heads, int kv_heads,
+                        int head_dim, float scale, int causal,
+                        const int *key_mask);
+
+/* ---- additions (no counterpart in the reference header) ---- */
+
+/* The Q and K calls that every reference call site issues back to back
+ * (e.g. iris_transformer_flux.c:3834-3837, iris_qwen3.c:1590-1593) as ONE
+ * launch: xq has q_heads heads normalised with wq, xk has k_heads heads
+ * normalised with wk; both share ld, the tables, eps and the pairing.
+ * Same result as the two iris_dev_head_norm_rope calls. */
+void iris_dev_head_norm_rope_qk(uint16_t *xq, uint16_t *xk, int ld,
+                                const float *wq, const float *wk,
+                                const float *rope_cos, const float *rope_sin,
+                                int seq, int q_heads, int k_heads, int head_dim,
+                                float eps, int split_half);
+
+/* The library's stream as a hipStream_t, for callers that time kernels with
+ * HIP events or order their own work after the library's. */
+void *iris_dev_stream(void);
+
+/* 0 when the most recent compute / memory entry succeeded, else a HIP error
+ * code or -1 for a rejected argument; reading it clears it. Lets a test see
+ * the failures that the void entries only report on stderr. */
+int iris_dev_last_error(void);
+
+/* Which kernel the most recent iris_dev_attention / iris_dev_head_norm_rope
+ * call used: a static string such as "fa_hd128" or "generic". */
+const char *iris_dev_last_kernel(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* IRIS_DEV_H */

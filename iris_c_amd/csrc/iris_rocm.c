@@ -1,0 +1,196 @@
+/*
+ * Host side of the MI355X backend: plain C over the HIP runtime C API.
+ * Owns the device state (one stream, device 0), the memory entries, and the
+ * argument checks that choose a kernel for the two hot-path operators. The
+ * kernels themselves live in the .hip files and are reached through the
+ * launchers of iris_kernels_hip.h.
+ *
+ * Behaviour follows the reference backend (iris_cuda.cu:108-230, 445-453,
+ * 878-937): compute entries never abort and never return a status; a failure
+ * is one line on stderr prefixed "iris_dev:". There is no CPU fallback: if
+ * the device is missing or the library was not initialised, the entries
+ * report the error and leave the output untouched.
+ */
+#define __HIP_PLATFORM_AMD__ 1
+#include <hip/hip_runtime_api.h>
+
+#include <stdio.h>
+#include <string.h>
+
+#include "iris_dev.h"
+#include "iris_kernels_hip.h"
+
+static int g_ready = 0;
+static char g_name[640] = "none";
+static hipStream_t g_stream = NULL;
+static int g_last_error = 0;
+static const char *g_last_kernel = "none";
+
+static void fail(int code, const char *what, const char *detail) {
+    g_last_error = code ? code : -1;
+    fprintf(stderr, "iris_dev: %s failed: %s\n", what, detail);
+}
+
+static int check(hipError_t err, const char *what) {
+    if (err == hipSuccess) return 1;
+    fail((int)err, what, hipGetErrorString(err));
+    return 0;
+}
+
+static int need_ready(const char *what) {
+    if (g_ready) return 1;
+    fail(-1, what, "device not initialised (iris_dev_init() did not succeed)");
+    return 0;
+}
+
+int iris_dev_init(void) {
+    if (g_ready) return 1;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count == 0) return 0;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, 0) != hipSuccess) return 0;
+    /* The kernels are compiled for gfx950 only. */
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        fprintf(stderr, "iris_dev: device 0 is %s, this backend needs gfx950\n", prop.gcnArchName);
+        return 0;
+    }
+    if (hipSetDevice(0) != hipSuccess) return 0;
+    snprintf(g_name, sizeof(g_name), "%s (%s, %d CUs)", prop.name, prop.gcnArchName,
+             prop.multiProcessorCount);
+    if (hipStreamCreate(&g_stream) != hipSuccess) return 0;
+    g_ready = 1;
+    g_last_error = 0;
+    return 1;
+}
+
+int iris_dev_available(void) { return g_ready; }
+const char *iris_dev_name(void) { return g_name; }
+void *iris_dev_stream(void) { return (void *)g_stream; }
+const char *iris_dev_last_kernel(void) { return g_last_kernel; }
+
+int iris_dev_last_error(void) {
+    int e = g_last_error;
+    g_last_error = 0;
+    return e;
+}
+
+void iris_dev_cleanup(void) {
+    if (!g_ready) return;
+    check(hipStreamSynchronize(g_stream), "sync");
+    check(hipStreamDestroy(g_stream), "stream destroy");
+    g_stream = NULL;
+    g_ready = 0;
+}
+
+void *iris_dev_alloc(size_t bytes) {
+    void *p = NULL;
+    if (!need_ready("alloc")) return NULL;
+    if (hipMalloc(&p, bytes ? bytes : 1) != hipSuccess) {
+        (void)hipGetLastError();
+        return NULL;
+    }
+    return p;
+}
+
+void iris_dev_free(void *p) {
+    if (!p || !need_ready("free")) return;
+    check(hipStreamSynchronize(g_stream), "sync");   /* pending work may still use the buffer */
+    check(hipFree(p), "free");
+}
+
+void iris_dev_upload_2d(void *dst, size_t dst_stride, const void *src, size_t src_stride,
+                        size_t row_bytes, size_t rows) {
+    if (!need_ready("upload") || !row_bytes || !rows) return;
+    check(hipMemcpy2DAsync(dst, dst_stride, src, src_stride, row_bytes, rows,
+                           hipMemcpyHostToDevice, g_stream), "upload");
+    check(hipStreamSynchronize(g_stream), "sync");
+}
+
+void iris_dev_upload(void *dst, const void *src, size_t bytes) {
+    if (!need_ready("upload") || !bytes) return;
+    check(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream), "upload");
+    check(hipStreamSynchronize(g_stream), "sync");
+}
+
+void iris_dev_download(void *dst, const void *src, size_t bytes) {
+    if (!need_ready("download")) return;
+    if (bytes) check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream), "download");
+    check(hipStreamSynchronize(g_stream), "sync");
+}
+
+void iris_dev_sync(void) {
+    if (!need_ready("sync")) return;
+    check(hipStreamSynchronize(g_stream), "sync");
+}
+
+static int aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+/* Shared by the one- and two-tensor entries; xk may be NULL with k_heads 0. */
+static void norm_rope(uint16_t *xq, uint16_t *xk, int ld, const float *wq, const float *wk,
+                      const float *rope_cos, const float *rope_sin, int seq, int q_heads,
+                      int k_heads, int head_dim, float eps, int split_half) {
+    if (!need_ready("head_norm_rope")) return;
+    if (seq <= 0 || q_heads + k_heads <= 0) return;
+    if (head_dim <= 0 || (head_dim & 1) || head_dim > 1024) {
+        fail(-1, "head_norm_rope", "head_dim must be even and <= 1024");
+        return;
+    }
+    int fast = head_dim == 128 && ld % 8 == 0 && aligned(xq, 16) && aligned(wq, 16) &&
+               aligned(rope_cos, 16) && aligned(rope_sin, 16) &&
+               (long long)seq * (q_heads + k_heads) < (1 << 24) && q_heads + k_heads < 256;
+    if (k_heads > 0) fast = fast && aligned(xk, 16) && aligned(wk, 16);
+    int err;
+    if (fast) {
+        g_last_kernel = "norm_rope_hd128";
+        err = iris_hip_norm_rope_hd128(g_stream, xq, xk, ld, wq, wk, rope_cos, rope_sin, seq,
+                                       q_heads, k_heads, eps, split_half != 0);
+    } else {
+        g_last_kernel = "norm_rope_generic";
+        err = iris_hip_norm_rope_generic(g_stream, xq, ld, wq, rope_cos, rope_sin, seq, q_heads,
+                                         head_dim, eps, split_half != 0);
+        if (!err && k_heads > 0)
+            err = iris_hip_norm_rope_generic(g_stream, xk, ld, wk, rope_cos, rope_sin, seq,
+                                             k_heads, head_dim, eps, split_half != 0);
+    }
+    if (err) check((hipError_t)err, "head_norm_rope launch");
+}
+
+void iris_dev_head_norm_rope(uint16_t *x, int ld, const float *w,
+                             const float *rope_cos, const float *rope_sin,
+                             int seq, int heads, int head_dim, float eps, int split_half) {
+    norm_rope(x, NULL, ld, w, NULL, rope_cos, rope_sin, seq, heads, 0, head_dim, eps, split_half);
+}
+
+void iris_dev_head_norm_rope_qk(uint16_t *xq, uint16_t *xk, int ld,
+                                const float *wq, const float *wk,
+                                const float *rope_cos, const float *rope_sin,
+                                int seq, int q_heads, int k_heads, int head_dim,
+                                float eps, int split_half) {
+    norm_rope(xq, xk, ld, wq, wk, rope_cos, rope_sin, seq, q_heads, k_heads, head_dim, eps,
+              split_half);
+}
+
+void iris_dev_attention(uint16_t *out, int ldo,
+                        const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                        int ldi, int seq_q, int seq_k, int heads, int kv_heads,
+                        int head_dim, float scale, int causal, const int *key_mask) {
+    if (!need_ready("attention")) return;
+    if (seq_q <= 0 || heads <= 0) return;
+    if (kv_heads <= 0 || heads % kv_heads != 0 || head_dim <= 0 || head_dim > 512 || seq_k < 0) {
+        fail(-1, "attention", "need heads % kv_heads == 0, 0 < head_dim <= 512, seq_k >= 0");
+        return;
+    }
+    int fast = head_dim == 128 && seq_k > 0 && scale > 0.0f && ldi % 8 == 0 && ldo % 4 == 0 &&
+               aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out, 8);
+    int err;
+    if (fast) {
+        g_last_kernel = "fa_hd128";
+        err = iris_hip_fa_hd128(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads,
+                                scale, causal != 0, key_mask);
+    } else {
+        g_last_kernel = "attention_generic";
+        err = iris_hip_attention_generic(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads,
+                                         kv_heads, head_dim, scale, causal != 0, key_mask);
+    }
+    if (err) check((hipError_t)err, "attention launch");
+}

@@ -1,0 +1,203 @@
+/*
+ * Fused per-head Q/K RMSNorm + rotary embedding for gfx950, in place on bf16.
+ *
+ * Semantics (reference iris_cuda.cu:402-420): for token s and head h, with
+ * v = x + s*ld + h*hd:  r = 1/sqrt(mean(v^2) + eps);  a = v[i0]*r*w[i0],
+ * b = v[i1]*r*w[i1];  v[i0] = a*c - b*sn, v[i1] = b*c + a*sn with
+ * (c, sn) = (cos, sin)[s*hd/2 + i] and (i0, i1) = (2i, 2i+1), or (i, i+hd/2)
+ * when split_half. f32 math, one round-to-nearest-even at the store.
+ *
+ * Mapping for head_dim 128 (the only size the models use): one (token, head)
+ * vector is 256 B = 16 lanes x 16 B, so a wave64 moves four vectors per
+ * 128-bit load/store and the four are contiguous in memory (heads of one
+ * token are adjacent). The sum of squares is reduced inside the 16-lane DPP
+ * row (row_ror 8/4/2/1), so there is no LDS and no barrier. Each wave keeps
+ * UNROLL independent vectors in flight. Q and K of the same rows can go in
+ * one launch: the unit index then runs over q_heads + k_heads per token.
+ *
+ * HBM traffic per vector: 256 B read + 256 B written; the cos/sin rows
+ * (512 B per token) are shared by all heads of the token and stay in L2.
+ */
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "iris_kernels_hip.h"
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;                       /* vectors in flight per 16-lane row */
+constexpr int kUnitsPerBlock = (kThreads / 16) * kUnroll;
+
+__device__ __forceinline__ float bf_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+
+/* Two f32 -> packed bf16x2, round to nearest even (v_cvt_pk_bf16_f32; equals
+ * the integer form u += 0x7fff + ((u >> 16) & 1) for every finite input). */
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    f32x2 p = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2));
+}
+
+/* Sum over the 16 lanes of a DPP row; every lane gets the total. */
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));
+    return v;
+}
+
+/* The value held by the lane 8 places away in the same 16-lane row. */
+__device__ __forceinline__ float row16_partner8(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
+}
+
+template <bool SPLIT>
+__global__ void __launch_bounds__(kThreads)
+k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
+                  const float *__restrict__ wq, const float *__restrict__ wk,
+                  const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
+                  int units, int q_heads, int heads_total, uint32_t magic, float eps) {
+    const int sub = threadIdx.x & 15;             /* which 16 B of the 256 B vector */
+    const int row = threadIdx.x >> 4;             /* 16-lane row inside the block */
+    const int first = blockIdx.x * kUnitsPerBlock + row;
+
+    /* Table columns this lane needs: consecutive pairs -> i = 4*sub..4*sub+3;
+     * split-half -> i = 8*(sub&7)..+7 (shared with the partner lane). */
+    const int tcol = SPLIT ? 8 * (sub & 7) : 4 * sub;
+    const float sgn = (SPLIT && sub < 8) ? -1.0f : 1.0f;
+
+    uint4 raw[kUnroll];
+    int tok[kUnroll];
+    uint16_t *ptr[kUnroll];
+    bool isk[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+        int unit = first + u * (kThreads / 16);
+        bool live = unit < units;
+        unit = live ? unit : 0;
+        int s = (int)__umulhi((uint32_t)unit, magic);       /* unit / heads_total */
+        int h = unit - s * heads_total;
+        isk[u] = h >= q_heads;
+        uint16_t *base = isk[u] ? xk + (size_t)(h - q_heads) * 128 : xq + (size_t)h * 128;
+        ptr[u] = live ? base + (size_t)s * ld + sub * 8 : nullptr;
+        tok[u] = s;
+        raw[u] = live ? *reinterpret_cast<const uint4 *>(ptr[u]) : make_uint4(0, 0, 0, 0);
+    }
+
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+        if (!ptr[u]) continue;
+        float e[8] = {bf_lo(raw[u].x), bf_hi(raw[u].x), bf_lo(raw[u].y), bf_hi(raw[u].y),
+                      bf_lo(raw[u].z), bf_hi(raw[u].z), bf_lo(raw[u].w), bf_hi(raw[u].w)};
+        float ss = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) ss = fmaf(e[i], e[i], ss);
+        ss = row16_sum(ss);
+        const float inv = 1.0f / sqrtf(ss * (1.0f / 128.0f) + eps);
+
+        const float *w = isk[u] ? wk : wq;
+        const float4 w0 = *reinterpret_cast<const float4 *>(w + sub * 8);
+        const float4 w1 = *reinterpret_cast<const float4 *>(w + sub * 8 + 4);
+        const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) e[i] *= inv * wv[i];
+
+        const float *cp = rope_cos + (size_t)tok[u] * 64 + tcol;
+        const float *sp = rope_sin + (size_t)tok[u] * 64 + tcol;
+        float o[8];
+        if (SPLIT) {
+            const float4 c0 = *reinterpret_cast<const float4 *>(cp);
+            const float4 c1 = *reinterpret_cast<const float4 *>(cp + 4);
+            const float4 s0 = *reinterpret_cast<const float4 *>(sp);
+            const float4 s1 = *reinterpret_cast<const float4 *>(sp + 4);
+            const float cv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+            const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                /* lanes 0-7 hold a (first half), lanes 8-15 hold b: a*c - b*s / b*c + a*s */
+                float other = row16_partner8(e[i]);
+                o[i] = fmaf(sgn * other, sv[i], e[i] * cv[i]);
+            }
+        } else {
+            const float4 c = *reinterpret_cast<const float4 *>(cp);
+            const float4 s = *reinterpret_cast<const float4 *>(sp);
+            const float cv[4] = {c.x, c.y, c.z, c.w};
+            const float sv[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                float a = e[2 * p], b = e[2 * p + 1];
+                o[2 * p] = fmaf(-b, sv[p], a * cv[p]);
+                o[2 * p + 1] = fmaf(a, sv[p], b * cv[p]);
+            }
+        }
+        uint4 out;
+        out.x = pack_bf16(o[0], o[1]);
+        out.y = pack_bf16(o[2], o[3]);
+        out.z = pack_bf16(o[4], o[5]);
+        out.w = pack_bf16(o[6], o[7]);
+        *reinterpret_cast<uint4 *>(ptr[u]) = out;
+    }
+}
+
+/* Any even head_dim: one wave per (token, head), lanes stride over pairs. */
+__global__ void __launch_bounds__(64)
+k_norm_rope_generic(uint16_t *x, int ld, const float *w, const float *rope_cos,
+                    const float *rope_sin, int heads, int head_dim, float eps, int split_half) {
+    const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int half = head_dim / 2;
+    uint16_t *v = x + (size_t)s * ld + (size_t)h * head_dim;
+    float ss = 0.0f;
+    for (int d = lane; d < head_dim; d += 64) {
+        float f = __uint_as_float((uint32_t)v[d] << 16);
+        ss = fmaf(f, f, ss);
+    }
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    const float inv = 1.0f / sqrtf(ss / (float)head_dim + eps);
+    for (int i = lane; i < half; i += 64) {
+        int i0 = split_half ? i : 2 * i, i1 = split_half ? i + half : 2 * i + 1;
+        float a = __uint_as_float((uint32_t)v[i0] << 16) * (inv * w[i0]);
+        float b = __uint_as_float((uint32_t)v[i1] << 16) * (inv * w[i1]);
+        float c = rope_cos[(size_t)s * half + i], sn = rope_sin[(size_t)s * half + i];
+        uint32_t packed = pack_bf16(fmaf(-b, sn, a * c), fmaf(a, sn, b * c));
+        v[i0] = (uint16_t)(packed & 0xffffu);
+        v[i1] = (uint16_t)(packed >> 16);
+    }
+}
+
+}  // namespace
+
+extern "C" int iris_hip_norm_rope_hd128(void *stream, uint16_t *xq, uint16_t *xk, int ld,
+                                        const float *wq, const float *wk,
+                                        const float *rope_cos, const float *rope_sin,
+                                        int seq, int q_heads, int k_heads, float eps,
+                                        int split_half) {
+    const int heads_total = q_heads + k_heads;
+    const int units = seq * heads_total;
+    if (units <= 0) return 0;
+    /* unit / heads_total == umulhi(unit, magic) for unit < 2^24, heads_total < 2^8 */
+    const uint32_t magic = (uint32_t)((0x100000000ull + heads_total - 1) / heads_total);
+    const int blocks = (units + kUnitsPerBlock - 1) / kUnitsPerBlock;
+    hipStream_t st = (hipStream_t)stream;
+    if (split_half)
+        hipLaunchKernelGGL(k_norm_rope_hd128<true>, dim3(blocks), dim3(kThreads), 0, st, xq, xk, ld,
+                           wq, wk, rope_cos, rope_sin, units, q_heads, heads_total, magic, eps);
+    else
+        hipLaunchKernelGGL(k_norm_rope_hd128<false>, dim3(blocks), dim3(kThreads), 0, st, xq, xk, ld,
+                           wq, wk, rope_cos, rope_sin, units, q_heads, heads_total, magic, eps);
+    return (int)hipGetLastError();
+}
+
+extern "C" int iris_hip_norm_rope_generic(void *stream, uint16_t *x, int ld, const float *w,
+                                          const float *rope_cos, const float *rope_sin,
+                                          int seq, int heads, int head_dim, float eps,
+                                          int split_half) {
+    if (seq <= 0 || heads <= 0) return 0;
+    hipLaunchKernelGGL(k_norm_rope_generic, dim3(seq, heads), dim3(64), 0, (hipStream_t)stream, x, ld,
+                       w, rope_cos, rope_sin, heads, head_dim, eps, split_half);
+    return (int)hipGetLastError();
+}

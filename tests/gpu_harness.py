@@ -1,0 +1,86 @@
+"""Runs the two operators through the C ABI on numpy inputs (GPU tests only)."""
+import ctypes as C
+
+import numpy as np
+
+_vp = C.c_void_p
+
+
+def ptr_add(p, nbytes):
+    return C.c_void_p((p if isinstance(p, int) else p.value if hasattr(p, "value") else int(p)) + nbytes)
+
+
+class Dev:
+    def __init__(self):
+        import iris_c_amd
+        self.dev = iris_c_amd.IrisDev()
+        self.lib = self.dev.lib
+        self._allocs = []
+
+    def put(self, arr):
+        p = self.dev.to_device(arr)
+        self._allocs.append(p)
+        return p
+
+    def alloc(self, nbytes):
+        p = self.lib.iris_dev_alloc(nbytes)
+        assert p, "iris_dev_alloc failed"
+        self._allocs.append(p)
+        return p
+
+    def get(self, p, shape, dtype):
+        return self.dev.to_host(p, shape, dtype)
+
+    def free_all(self):
+        for p in self._allocs:
+            self.lib.iris_dev_free(p)
+        self._allocs = []
+
+    def check(self):
+        self.dev.check()
+
+    def norm_rope(self, buf, ld, col0, w, cos, sin, seq, heads, hd, eps, split_half):
+        """In place on a host uint16 buffer image; returns the new buffer."""
+        d = self.put(buf)
+        dw, dc, ds = self.put(w.astype(np.float32)), self.put(cos.astype(np.float32)), self.put(sin.astype(np.float32))
+        self.lib.iris_dev_head_norm_rope(ptr_add(d, 2 * col0), ld, dw, dc, ds, seq, heads, hd, eps, split_half)
+        self.check()
+        out = self.get(d, buf.shape, np.uint16)
+        self.free_all()
+        return out
+
+    def norm_rope_qk(self, buf, ld, qcol, kcol, wq, wk, cos, sin, seq, q_heads, k_heads, hd, eps, split_half):
+        d = self.put(buf)
+        dwq, dwk = self.put(wq.astype(np.float32)), self.put(wk.astype(np.float32))
+        dc, ds = self.put(cos.astype(np.float32)), self.put(sin.astype(np.float32))
+        self.lib.iris_dev_head_norm_rope_qk(ptr_add(d, 2 * qcol), ptr_add(d, 2 * kcol), ld, dwq, dwk, dc, ds,
+                                            seq, q_heads, k_heads, hd, eps, split_half)
+        self.check()
+        out = self.get(d, buf.shape, np.uint16)
+        self.free_all()
+        return out
+
+    def attention(self, buf, ldi, qcol, kcol, vcol, seq_q, seq_k, heads, kv_heads, hd, scale, causal=False,
+                  key_mask=None, ldo=None, out_col=0, out_fill=0x7fc0):
+        """Returns the bf16 output rows as uint16 [seq_q, ldo]."""
+        ldo = ldo or heads * hd
+        d = self.put(buf)
+        out0 = np.full((max(seq_q, 1), ldo), out_fill, dtype=np.uint16)
+        do = self.put(out0)
+        dm = self.put(np.ascontiguousarray(key_mask, dtype=np.int32)) if key_mask is not None else None
+        self.lib.iris_dev_attention(ptr_add(do, 2 * out_col), ldo, ptr_add(d, 2 * qcol), ptr_add(d, 2 * kcol),
+                                    ptr_add(d, 2 * vcol), ldi, seq_q, seq_k, heads, kv_heads, hd, scale,
+                                    int(causal), dm)
+        self.check()
+        kernel = self.dev.last_kernel()
+        out = self.get(do, out0.shape, np.uint16)
+        self.free_all()
+        return out, kernel
+
+
+def error_stats(got, want):
+    diff = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    return float(diff.max()), float(diff.mean())
+
+
+MAX_ABS, MEAN_ABS = 2e-2, 2e-3      # bf16 device output vs fp32 CPU oracle on identical inputs

@@ -1,0 +1,67 @@
+"""The C-ABI library: builds in-tree, exports every symbol include/iris_dev.h
+declares, and behaves sanely without a GPU (no compute is attempted here)."""
+import os
+import re
+
+import pytest
+
+import iris_c_amd
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(iris_c_amd.LIB_PATH):
+        iris_c_amd.build()
+    return iris_c_amd.load()
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "iris_dev.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"\b(iris_dev_\w+)\s*\(", text)
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    names = declared_functions()
+    assert len(names) >= 14
+    assert set(names) == set(iris_c_amd.ABI), set(names) ^ set(iris_c_amd.ABI)
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
+def test_reference_signatures_are_kept():
+    """Argument lists of the two hot-path entries, as the reference header declares them."""
+    text = re.sub(r"\s+", " ", open(os.path.join(ROOT, "include", "iris_dev.h")).read())
+    assert ("void iris_dev_head_norm_rope(uint16_t *x, int ld, const float *w, const float *rope_cos, "
+            "const float *rope_sin, int seq, int heads, int head_dim, float eps, int split_half);") in text
+    assert ("void iris_dev_attention(uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k, "
+            "const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads, int head_dim, "
+            "float scale, int causal, const int *key_mask);") in text
+
+
+def test_no_gpu_means_no_silent_fallback(lib):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    assert lib.iris_dev_init() == 0
+    assert lib.iris_dev_available() == 0
+    assert lib.iris_dev_alloc(16) is None
+    lib.iris_dev_last_error()
+    # compute entries refuse to run (and say so) instead of computing on the CPU
+    lib.iris_dev_attention(None, 0, None, None, None, 0, 4, 4, 1, 1, 128, 1.0, 0, None)
+    assert lib.iris_dev_last_error() != 0
+    lib.iris_dev_head_norm_rope(None, 0, None, None, None, 4, 1, 128, 1e-6, 0)
+    assert lib.iris_dev_last_error() != 0
+
+
+def test_product_does_not_link_the_oracle(lib):
+    import subprocess
+    out = subprocess.run(["ldd", iris_c_amd.LIB_PATH], capture_output=True, text=True).stdout
+    assert "oracle" not in out and "iris_ref" not in out
+    for root, _, files in os.walk(os.path.join(ROOT, "iris_c_amd")):
+        for f in files:
+            if f.endswith((".c", ".h", ".hip", ".py")):
+                src = open(os.path.join(root, f)).read()
+                assert "import oracle" not in src and "iris_oracle.h" not in src and "orc_" not in src, f

@@ -1,0 +1,224 @@
+"""iris_dev_attention on the GPU (through the C ABI) against the fp32 CPU
+oracle on identical bf16 inputs. Bar: max-abs <= 2e-2, mean-abs <= 2e-3.
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+import workloads as W
+from gpu_harness import Dev, error_stats, MAX_ABS, MEAN_ABS
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    return Dev()
+
+
+def gpu_attention(dev, case, **over):
+    a = dict(case); a.update(over)
+    out, kernel = dev.attention(a["buf"], a["ldi"], 0, a["q_dim"], a["q_dim"] + a["kv_dim"], a["seq"], a["seq"],
+                                a["heads"], a["kv_heads"], 128, a["scale"], a["causal"], a["key_mask"], ldo=a["ldo"])
+    return O.bf16_to_f32(out[:, :a["q_dim"]]), kernel
+
+
+def cpu_attention(orc, case, rows=None):
+    return orc.attention_bf16(case["buf"], case["ldi"], 0, case["q_dim"], case["q_dim"] + case["kv_dim"], case["seq"],
+                              case["seq"], case["heads"], case["kv_heads"], 128, case["scale"], case["causal"],
+                              case["key_mask"], rows=rows)
+
+
+def assert_close(got, want, what=""):
+    mx, mean = error_stats(got, want)
+    assert mx <= MAX_ABS and mean <= MEAN_ABS, f"{what}: max-abs {mx:.4g}, mean-abs {mean:.4g}"
+    return mx, mean
+
+
+def after_norm_rope(dev, case):
+    """The caller's sequence: norm+rope on Q, on K, then attention."""
+    buf = dev.norm_rope_qk(case["buf"], case["ldi"], 0, case["q_dim"], case["wq"], case["wk"], case["cos"], case["sin"],
+                           case["seq"], case["heads"], case["kv_heads"], 128, case["eps"], case["split_half"])
+    out = dict(case); out["buf"] = buf
+    return out
+
+
+# ------------------------------------------------------------------ the five configurations, shrunk
+def test_c1_plumbing_full_size(dev, orc):
+    case = after_norm_rope(dev, W.c1())           # 64 text + 16x16 image, 24 heads
+    got, kernel = gpu_attention(dev, case)
+    assert kernel == "fa_hd128"
+    assert_close(got, cpu_attention(orc, case), "C1")
+    # and against the reference-shaped f32 flash attention on the same inputs
+    f = O.bf16_to_f32(case["buf"])
+    flash = orc.attention_flash(f[:, :3072], f[:, 3072:6144], f[:, 6144:], 24, case["scale"])
+    assert_close(got, flash, "C1 vs flash")
+
+
+@pytest.mark.parametrize("maker,shrink", [(W.c2, 8), (W.c5, 32)])
+def test_joint_attention_shrunk(dev, orc, maker, shrink):
+    case = after_norm_rope(dev, maker(shrink))
+    got, kernel = gpu_attention(dev, case)
+    assert kernel == "fa_hd128"
+    assert_close(got, cpu_attention(orc, case), case["name"])
+
+
+def test_c3_cfg_pair_with_key_mask(dev, orc):
+    for case in W.c3(shrink=8):
+        case = after_norm_rope(dev, case)
+        got, kernel = gpu_attention(dev, case)
+        assert kernel == "fa_hd128"
+        assert_close(got, cpu_attention(orc, case), case["name"])
+
+
+@pytest.mark.parametrize("shrink", [1, 4])
+def test_c4_causal_gqa_padding(dev, orc, shrink):
+    case = after_norm_rope(dev, W.c4(shrink))
+    got, kernel = gpu_attention(dev, case)
+    assert kernel == "fa_hd128"
+    assert_close(got, cpu_attention(orc, case), "C4")
+
+
+# ------------------------------------------------------------------ full sizes: sampled rows + properties
+def sample_rows(seq, n=40, seed=0):
+    rng = np.random.default_rng(seed)
+    fixed = [0, 1, 127, 128, 511, 512, seq // 2, seq - 129, seq - 128, seq - 1]
+    return np.unique(np.r_[fixed, rng.integers(0, seq, n)]).astype(np.int32)
+
+
+def test_c2_full_size_sampled_rows_and_properties(dev, orc):
+    case = after_norm_rope(dev, W.c2())
+    got, kernel = gpu_attention(dev, case)
+    assert kernel == "fa_hd128"
+    rows = sample_rows(case["seq"])
+    assert_close(got[rows], cpu_attention(orc, case, rows=rows), "C2 sampled")
+    # key-permutation invariance (non-causal): shuffle K/V rows together
+    perm = np.random.default_rng(1).permutation(case["seq"])
+    shuf = case["buf"].copy()
+    shuf[:, 3072:] = case["buf"][perm][:, 3072:]
+    got2, _ = gpu_attention(dev, case, buf=shuf)
+    assert_close(got2, got, "C2 permuted keys")
+    # constant V -> every output row equals that V row
+    const = case["buf"].copy()
+    const[:, 6144:] = case["buf"][7, 6144:]
+    got3, _ = gpu_attention(dev, case, buf=const)
+    want = np.tile(O.bf16_to_f32(case["buf"][7, 6144:]), (case["seq"], 1))
+    assert_close(got3, want, "C2 constant V")
+
+
+def test_c5_full_size_sampled_rows(dev, orc):
+    case = after_norm_rope(dev, W.c5())           # 12800 tokens
+    got, kernel = gpu_attention(dev, case)
+    assert kernel == "fa_hd128"
+    rows = sample_rows(case["seq"], n=20)
+    assert_close(got[rows], cpu_attention(orc, case, rows=rows), "C5 sampled")
+
+
+def test_c3_full_size_masked_equals_compacted(dev, orc):
+    cond, unc = W.c3()
+    unc = after_norm_rope(dev, unc)
+    got, _ = gpu_attention(dev, unc)
+    rows = sample_rows(unc["seq"], n=20)
+    assert_close(got[rows], cpu_attention(orc, unc, rows=rows), "C3 uncond sampled")
+    # masked keys == the same problem with those K/V rows removed
+    keep = np.nonzero(unc["key_mask"])[0]
+    small = dict(unc); small["buf"] = np.ascontiguousarray(unc["buf"][keep]); small["seq"] = keep.size; small["key_mask"] = None
+    got_small, _ = gpu_attention(dev, small)
+    assert_close(got[keep], got_small, "C3 masked vs compacted")
+
+
+# ------------------------------------------------------------------ edge cases
+def random_case(seed, seq_q, seq_k, heads, kv_heads, hd=128, pad=0, sigma=1.0):
+    rng = np.random.default_rng(seed)
+    seq = max(seq_q, seq_k)
+    ldi = (heads + 2 * kv_heads) * hd + pad
+    buf = O.f32_to_bf16(rng.standard_normal((seq, ldi)).astype(np.float32) * sigma)
+    return buf, ldi
+
+
+@pytest.mark.parametrize("seq_q,seq_k", [(1, 1), (1, 64), (5, 63), (33, 65), (128, 128), (129, 191), (200, 31), (257, 1000)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_ragged_shapes(dev, orc, seq_q, seq_k, causal):
+    heads, kv = 4, 2
+    buf, ldi = random_case(seq_q * 7 + seq_k, seq_q, seq_k, heads, kv)
+    qd, kd = heads * 128, kv * 128
+    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, 128, 0.0884, causal)
+    assert kernel == "fa_hd128"
+    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, 128, 0.0884, causal)
+    assert_close(O.bf16_to_f32(out[:seq_q]), want, f"{seq_q}x{seq_k} causal={causal}")
+
+
+def test_random_key_masks_and_empty_rows(dev, orc):
+    heads, seq = 3, 300
+    buf, ldi = random_case(5, seq, seq, heads, heads)
+    rng = np.random.default_rng(6)
+    mask = (rng.random(seq) < 0.5).astype(np.int32)
+    out, _ = dev.attention(buf, ldi, 0, 384, 768, seq, seq, heads, heads, 128, 0.0884, False, mask)
+    want = orc.attention_bf16(buf, ldi, 0, 384, 768, seq, seq, heads, heads, 128, 0.0884, False, mask)
+    assert_close(O.bf16_to_f32(out), want, "random mask")
+    # causal + mask whose first valid key is 10: queries 0..9 have no valid key -> zero rows
+    mask2 = np.ones(seq, np.int32); mask2[:10] = 0
+    out, _ = dev.attention(buf, ldi, 0, 384, 768, seq, seq, heads, heads, 128, 0.0884, True, mask2)
+    got = O.bf16_to_f32(out)
+    assert np.all(got[:10] == 0.0)
+    want = orc.attention_bf16(buf, ldi, 0, 384, 768, seq, seq, heads, heads, 128, 0.0884, True, mask2)
+    assert_close(got[10:], want[10:], "causal + mask")
+    # all keys masked -> all-zero output
+    out, _ = dev.attention(buf, ldi, 0, 384, 768, seq, seq, heads, heads, 128, 0.0884, False, np.zeros(seq, np.int32))
+    assert np.all(O.bf16_to_f32(out) == 0.0)
+
+
+def test_large_scores_stay_finite(dev, orc):
+    heads, seq = 2, 130
+    buf, ldi = random_case(9, seq, seq, heads, heads, sigma=6.0)     # |score| up to ~100
+    out, _ = dev.attention(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, 0.0884)
+    got = O.bf16_to_f32(out)
+    assert np.all(np.isfinite(got))
+    want = orc.attention_bf16(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, 0.0884)
+    mx, mean = error_stats(got, want)
+    assert mx <= 0.13 and mean <= 4e-3      # outputs are O(6): same relative bar as 2e-2 on O(1) values
+
+
+def test_output_stride_and_interior_pointers(dev, orc):
+    heads, seq = 2, 70
+    buf, ldi = random_case(11, seq, seq, heads, heads, pad=64)
+    ldo, out_col = 2 * 256 + 8, 256
+    out, kernel = dev.attention(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, 0.0884, ldo=ldo, out_col=out_col)
+    assert kernel == "fa_hd128"
+    want = orc.attention_bf16(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, 0.0884)
+    assert_close(O.bf16_to_f32(out[:, out_col:out_col + 256]), want, "strided out")
+    assert np.all(out[:, :out_col] == 0x7fc0) and np.all(out[:, out_col + 256:] == 0x7fc0)
+
+
+@pytest.mark.parametrize("hd,heads,kv,causal,masked", [(64, 4, 4, False, False), (64, 4, 2, True, True),
+                                                       (512, 1, 1, False, False), (96, 2, 1, True, False)])
+def test_generic_kernel_other_head_dims(dev, orc, hd, heads, kv, causal, masked):
+    seq = 150
+    buf, ldi = random_case(hd + heads, seq, seq, heads, kv, hd=hd)
+    qd, kd = heads * hd, kv * hd
+    mask = None
+    if masked:
+        mask = (np.arange(seq) < 101).astype(np.int32)
+    scale = 1 / np.sqrt(hd)
+    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq, seq, heads, kv, hd, scale, causal, mask)
+    assert kernel == "attention_generic"
+    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq, seq, heads, kv, hd, scale, causal, mask)
+    assert_close(O.bf16_to_f32(out), want, f"generic hd={hd}")
+
+
+def test_misaligned_stride_falls_back_not_fails(dev, orc):
+    heads, seq = 2, 40
+    buf, ldi = random_case(13, seq, seq, heads, heads, pad=3)      # ldi % 8 != 0
+    out, kernel = dev.attention(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, 0.0884)
+    assert kernel == "attention_generic"
+    want = orc.attention_bf16(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, 0.0884)
+    assert_close(O.bf16_to_f32(out), want, "misaligned")
+
+
+def test_bad_arguments_are_reported_not_fatal(dev):
+    buf, ldi = random_case(1, 8, 8, 3, 2)
+    d = dev.put(buf)
+    dev.lib.iris_dev_last_error()
+    dev.lib.iris_dev_attention(d, 384, d, d, d, ldi, 8, 8, 3, 2, 128, 0.1, 0, None)    # 3 % 2 != 0
+    assert dev.lib.iris_dev_last_error() != 0
+    dev.free_all()
