@@ -19,7 +19,11 @@ HIP_SRCS = $(CSRC)/qknorm_rope.hip $(CSRC)/fa_fwd_gfx950.hip $(CSRC)/attn_generi
 HIP_OBJS = $(HIP_SRCS:.hip=.o)
 
 .PHONY: rocm oracle clean test-cpu test-gpu bench
-rocm: $(OUT)
+rocm: $(OUT) iris_c_amd/libiris_microbench.so
+
+# machine-ceiling microbenchmarks used by bench.py only
+iris_c_amd/libiris_microbench.so: $(CSRC)/microbench.hip
+	$(HIPCC) $(HIPFLAGS) -shared -o $@ $<
 
 $(CSRC)/%.o: $(CSRC)/%.hip $(CSRC)/iris_kernels_hip.h
 	$(HIPCC) $(HIPFLAGS) -c $< -o $@
@@ -41,4 +45,4 @@ bench:
 	python bench.py
 
 clean:
-	rm -f $(CSRC)/*.o $(OUT)
+	rm -f $(CSRC)/*.o $(OUT) iris_c_amd/libiris_microbench.so

@@ -1,0 +1,322 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+A step is what every transformer block of the reference issues for one
+sequence: fused per-head RMSNorm + RoPE on Q, on K, then joint attention
+(reference iris_transformer_flux.c:3834-3839), on the 24 heads x 128,
+512 text + 4096 image token configuration, bf16, inputs resident in HBM.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-shapes]
+
+Prints ONE JSON line. `value` is attention TFLOP/s over the whole step
+(algorithmic attention FLOPs / wall time of the triple). `roofline` is the
+attention kernel alone, timed with HIP events on the library's stream.
+`norm_rope` reports the bandwidth-bound kernel the same way. `shapes` lists
+latency / TFLOP/s / GB/s for every benchmark configuration. `cpu_baseline`
+times the reference's BLAS-build CPU structure on this host's cores.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 matrix peak (vendor figure)
+PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E peak
+
+_vp = C.c_void_p
+
+
+# ----------------------------------------------------------------------------- inputs
+def to_bf16(x):
+    """float32 ndarray -> uint16 bf16 patterns, round to nearest even."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def rope_table(pos_axes, dims, theta):
+    """cos/sin [seq, sum(dims)/2] for integer positions per axis (closed form)."""
+    cs, sn = [], []
+    for p, d in zip(pos_axes, dims):
+        freq = (1.0 / np.power(np.float32(theta), np.arange(0, d, 2, dtype=np.float32) / np.float32(d))).astype(np.float32)
+        ang = p.astype(np.float32)[:, None] * freq[None, :]
+        cs.append(np.cos(ang)); sn.append(np.sin(ang))
+    return np.concatenate(cs, 1).astype(np.float32), np.concatenate(sn, 1).astype(np.float32)
+
+
+def flux2_positions(txt, grid, refs):
+    img = grid * grid
+    seq = txt + img * (1 + refs)
+    T, H, Wd, L = (np.zeros(seq, np.int32) for _ in range(4))
+    L[:txt] = np.arange(txt)
+    ys, xs = np.divmod(np.arange(img), grid)
+    for i in range(1 + refs):
+        sl = slice(txt + i * img, txt + (i + 1) * img)
+        H[sl], Wd[sl], T[sl] = ys, xs, 10 * i
+    return [T, H, Wd, L]
+
+
+def make_config(name, rng):
+    """Synthetic data of one benchmark configuration (numpy PCG64 normals)."""
+    hd = 128
+    c = dict(name=name, hd=hd, causal=False, key_mask=None, split_half=0, eps=1e-6)
+    if name in ("C1", "C2", "C5"):
+        txt, grid, refs, sigma = {"C1": (64, 16, 0, 1.0), "C2": (512, 64, 0, 1 / np.sqrt(128)), "C5": (512, 64, 2, 1.0)}[name]
+        c.update(heads=24, kv_heads=24, seq=txt + grid * grid * (1 + refs), sigma=[sigma])
+        c["cos"], c["sin"] = rope_table(flux2_positions(txt, grid, refs), [32, 32, 32, 32], 2000.0)
+    elif name in ("C3-cond", "C3-uncond"):
+        seq = 4096 + 256
+        c.update(heads=30, kv_heads=30, seq=seq, eps=1e-5, sigma=[1 / np.sqrt(128)] if name == "C3-cond" else [0.1])
+        pos = [np.r_[np.full(4096, 257), 1 + np.arange(256)], np.r_[np.arange(4096) // 64, np.zeros(256)],
+               np.r_[np.arange(4096) % 64, np.zeros(256)]]
+        c["cos"], c["sin"] = rope_table([p.astype(np.int32) for p in pos], [32, 48, 48], 256.0)
+        if name == "C3-uncond":
+            length = int(rng.integers(16, 257))
+            c["key_mask"] = np.r_[np.ones(4096), np.arange(256) < length].astype(np.int32)
+    elif name == "C4":
+        seq = 512
+        c.update(heads=32, kv_heads=8, seq=seq, causal=True, split_half=1, sigma=[1.0])
+        c["cos"], c["sin"] = rope_table([np.arange(seq, dtype=np.int32)], [128], 1e6)
+        c["key_mask"] = (np.arange(seq) < int(rng.integers(8, 513))).astype(np.int32)
+    else:
+        raise ValueError(name)
+    c["q_dim"], c["kv_dim"] = c["heads"] * hd, c["kv_heads"] * hd
+    c["ldi"] = c["q_dim"] + 2 * c["kv_dim"]
+    c["ldo"] = c["q_dim"]
+    c["scale"] = float(1.0 / np.sqrt(np.float32(hd)))
+    buf = rng.standard_normal((c["seq"], c["ldi"]), dtype=np.float32) * np.float32(c["sigma"][0])
+    c["buf"] = to_bf16(buf)
+    c["wq"] = (1 + 0.02 * rng.standard_normal(hd)).astype(np.float32)
+    c["wk"] = (1 + 0.02 * rng.standard_normal(hd)).astype(np.float32)
+    return c
+
+
+def attention_flops(c):
+    valid = np.ones(c["seq"], np.int64) if c["key_mask"] is None else (c["key_mask"] != 0).astype(np.int64)
+    per_query = np.cumsum(valid) if c["causal"] else np.full(c["seq"], valid.sum())
+    return 4 * c["hd"] * c["heads"] * int(per_query.sum())
+
+
+def norm_rope_bytes(seq, heads, hd=128):
+    return 4 * seq * heads * hd + 2 * seq * (hd // 2) * 4 + hd * 4
+
+
+# ----------------------------------------------------------------------------- device plumbing
+class Hip:
+    """The few HIP runtime calls the timing needs (events on the library's stream)."""
+
+    def __init__(self):
+        self.rt = C.CDLL("libamdhip64.so")
+        self.rt.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), _vp, _vp]
+        self.rt.hipEventRecord.argtypes = [_vp, _vp]
+        self.rt.hipEventSynchronize.argtypes = [_vp]
+
+    def event(self):
+        ev = _vp()
+        assert self.rt.hipEventCreate(C.byref(ev)) == 0
+        return ev
+
+    def record(self, ev, stream):
+        assert self.rt.hipEventRecord(ev, stream) == 0
+
+    def elapsed_ms(self, a, b):
+        assert self.rt.hipEventSynchronize(b) == 0
+        ms = C.c_float()
+        assert self.rt.hipEventElapsedTime(C.byref(ms), a, b) == 0
+        return float(ms.value)
+
+
+class Resident:
+    """One configuration's tensors in HBM, `copies` rotating row buffers."""
+
+    def __init__(self, dev, c, copies):
+        self.c, self.dev, self.lib = c, dev, dev.lib
+        self.bufs = [dev.to_device(c["buf"]) for _ in range(copies)]
+        self.out = self.lib.iris_dev_alloc(c["seq"] * c["ldo"] * 2)
+        self.wq, self.wk = dev.to_device(c["wq"]), dev.to_device(c["wk"])
+        self.cos, self.sin = dev.to_device(c["cos"]), dev.to_device(c["sin"])
+        self.mask = dev.to_device(c["key_mask"]) if c["key_mask"] is not None else None
+        assert self.out and all(self.bufs)
+
+    def col(self, i, elems):
+        return _vp(self.bufs[i % len(self.bufs)] + 2 * elems)
+
+    def norm_q(self, i):
+        c = self.c
+        self.lib.iris_dev_head_norm_rope(self.col(i, 0), c["ldi"], self.wq, self.cos, self.sin, c["seq"], c["heads"],
+                                         c["hd"], c["eps"], c["split_half"])
+
+    def norm_k(self, i):
+        c = self.c
+        self.lib.iris_dev_head_norm_rope(self.col(i, c["q_dim"]), c["ldi"], self.wk, self.cos, self.sin, c["seq"],
+                                         c["kv_heads"], c["hd"], c["eps"], c["split_half"])
+
+    def norm_qk(self, i):
+        c = self.c
+        self.lib.iris_dev_head_norm_rope_qk(self.col(i, 0), self.col(i, c["q_dim"]), c["ldi"], self.wq, self.wk, self.cos,
+                                            self.sin, c["seq"], c["heads"], c["kv_heads"], c["hd"], c["eps"], c["split_half"])
+
+    def attention(self, i):
+        c = self.c
+        self.lib.iris_dev_attention(self.out, c["ldo"], self.col(i, 0), self.col(i, c["q_dim"]),
+                                    self.col(i, c["q_dim"] + c["kv_dim"]), c["ldi"], c["seq"], c["seq"], c["heads"],
+                                    c["kv_heads"], c["hd"], c["scale"], int(c["causal"]), self.mask)
+
+    def step(self, i):
+        """The caller's triple, as the reference models issue it (two norm calls, one attention)."""
+        self.norm_q(i); self.norm_k(i); self.attention(i)
+
+    def free(self):
+        for p in self.bufs + [self.out, self.wq, self.wk, self.cos, self.sin] + ([self.mask] if self.mask else []):
+            self.lib.iris_dev_free(p)
+
+
+def event_time(hip, stream, fn, reps, start=0):
+    """Average ms of `fn(i)` over `reps` back-to-back launches between two events."""
+    a, b = hip.event(), hip.event()
+    hip.record(a, stream)
+    for i in range(reps):
+        fn(start + i)
+    hip.record(b, stream)
+    return hip.elapsed_ms(a, b) / reps
+
+
+def per_launch_times(hip, stream, fn, reps):
+    """Per-launch ms with an event pair around every launch (for kernels >> event cost)."""
+    evs = [(hip.event(), hip.event()) for _ in range(reps)]
+    for i, (a, b) in enumerate(evs):
+        hip.record(a, stream); fn(i); hip.record(b, stream)
+    return [hip.elapsed_ms(a, b) for a, b in evs]
+
+
+# ----------------------------------------------------------------------------- CPU baseline
+def cpu_baseline(c):
+    """The reference's BLAS-build CPU attention (heads over pthreads, per head
+    sgemm -> softmax -> sgemm) on the same configuration, f32, on this host."""
+    import oracle
+    base = oracle.cpu_baseline()
+    f = (c["buf"].astype(np.uint32) << 16).view(np.float32)
+    q = np.ascontiguousarray(f[:, :c["q_dim"]])
+    k = np.ascontiguousarray(f[:, c["q_dim"]:c["q_dim"] + c["kv_dim"]])
+    v = np.ascontiguousarray(f[:, c["q_dim"] + c["kv_dim"]:])
+    cores = base.online_cpus()
+    box_share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    limit = min(cores, box_share) if box_share > 0 else cores
+    t0 = time.perf_counter()
+    _, threads = base.attention(q, k, v, c["heads"], c["kv_heads"], c["scale"], c["causal"], c["key_mask"],
+                                q_chunk=0, threads=limit)
+    dt = time.perf_counter() - t0
+    flops = attention_flops(c)
+    x = np.ascontiguousarray(q.reshape(c["seq"], c["heads"], c["hd"]))
+    t1 = time.perf_counter()
+    base.norm_rope(x, c["wq"], c["cos"], c["sin"], c["eps"], c["split_half"])
+    dn = time.perf_counter() - t1
+    return {"value": round(flops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"one full {c['name']} attention call ({c['heads']}h x {c['seq']} tok, f32), {dt:.2f} s; "
+                      f"sgemm from {os.path.basename(base.provider)}; host has {cores} CPUs online",
+            "attention_seconds": round(dt, 3),
+            "norm_rope_gbps": round(2 * x.nbytes / dn / 1e9, 3), "norm_rope_cores": 1}
+
+
+# ----------------------------------------------------------------------------- main
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-shapes", action="store_true", help="skip the per-configuration table")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (heads are independent, so the path would shard by "
+                 "head with no exchange); run with --gpus 1")
+
+    import iris_c_amd
+    dev = iris_c_amd.IrisDev()            # raises if the HIP library is missing or no gfx950 GPU
+    lib, hip = dev.lib, Hip()
+    stream = lib.iris_dev_stream()
+    rng = np.random.default_rng(20250101)
+
+    c2 = make_config("C2", rng)
+    copies = 8                             # 8 x 85 MB rows > 256 MB Infinity Cache: norm+rope reads come from HBM
+    res = Resident(dev, c2, copies)
+    flops = attention_flops(c2)
+
+    for i in range(args.warmup):
+        res.step(i)
+    lib.iris_dev_sync()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        res.step(i)
+    lib.iris_dev_sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    dev.check()
+
+    # dominant kernel alone: events around every attention launch
+    att = per_launch_times(hip, stream, res.attention, max(args.steps, 10))
+    att_ms = float(np.mean(att))
+    # bandwidth-bound kernel: back-to-back launches over rotating buffers (cold) and one buffer (warm)
+    reps = max(args.steps, 2 * copies)
+    nr_q_ms = event_time(hip, stream, res.norm_q, reps)
+    nr_qk_ms = event_time(hip, stream, res.norm_qk, reps)
+    nr_warm_ms = event_time(hip, stream, lambda i: res.norm_q(0), reps)
+    q_bytes = norm_rope_bytes(c2["seq"], c2["heads"])
+    qk_bytes = q_bytes + norm_rope_bytes(c2["seq"], c2["kv_heads"])
+    dev.check()
+
+    out = {
+        "metric": "joint_attention_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "C2: norm+rope(Q), norm+rope(K), joint attention; 24 heads x 128, 512 text + 4096 image "
+                               "tokens, fused qkv rows (ldi 9216), one sequence",
+                   "device": dev.name()},
+        "roofline": {"kernel": "k_fa_fwd_hd128", "bound": "mfma", "achieved": round(flops / (att_ms * 1e-3) / 1e12, 2),
+                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / (att_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+                     "traffic": None, "launch_ms": round(att_ms, 4), "launch_ms_min": round(float(np.min(att)), 4),
+                     "flops_per_launch": flops},
+        "norm_rope": {"kernel": "k_norm_rope_hd128", "bound": "hbm", "unit": "GB/s", "peak": PEAK_HBM_GBPS,
+                      "bytes_per_call": q_bytes,
+                      "q_call_us": round(nr_q_ms * 1e3, 2), "q_call_gbps": round(q_bytes / (nr_q_ms * 1e-3) / 1e9, 1),
+                      "q_call_frac": round(q_bytes / (nr_q_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                      "qk_fused_us": round(nr_qk_ms * 1e3, 2), "qk_fused_gbps": round(qk_bytes / (nr_qk_ms * 1e-3) / 1e9, 1),
+                      "qk_fused_frac": round(qk_bytes / (nr_qk_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                      "warm_cache_q_call_us": round(nr_warm_ms * 1e3, 2),
+                      "note": "cold = 8 rotating 85 MB row buffers (> 256 MB Infinity Cache); warm = same buffer every call"},
+    }
+    res.free()
+
+    if not args.no_shapes:
+        shapes = []
+        for name in ("C1", "C2", "C3-cond", "C3-uncond", "C4", "C5"):
+            c = c2 if name == "C2" else make_config(name, rng)
+            r = Resident(dev, c, 2)
+            for i in range(3):
+                r.step(i)
+            n = 20
+            a_ms = float(np.mean(per_launch_times(hip, stream, r.attention, n)))
+            qk_ms = event_time(hip, stream, r.norm_qk, n)
+            fl = attention_flops(c)
+            nb = norm_rope_bytes(c["seq"], c["heads"]) + norm_rope_bytes(c["seq"], c["kv_heads"])
+            shapes.append({"config": name, "seq": c["seq"], "heads": c["heads"], "kv_heads": c["kv_heads"],
+                           "attention_ms": round(a_ms, 4), "attention_tflops": round(fl / a_ms / 1e9, 2),
+                           "attention_frac_of_mfma_peak": round(fl / a_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                           "norm_rope_qk_us": round(qk_ms * 1e3, 2), "norm_rope_qk_gbps": round(nb / qk_ms / 1e6, 1)})
+            dev.check()
+            r.free()
+        out["shapes"] = shapes
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(c2)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -13,9 +13,9 @@
  * Shape of the computation on CDNA4
  * ---------------------------------
  * One workgroup = 4 waves = 128 queries of one head; each wave owns 32
- * queries for the whole kernel. Keys/values stream through LDS in tiles of
- * 64, the next tile travelling HBM -> registers while the current one is
- * being multiplied.
+ * queries for the whole kernel. Keys/values stream through two LDS stages in
+ * tiles of 64: while tile i is multiplied, tile i+1 moves registers -> LDS
+ * and tile i+2 moves HBM -> registers; one barrier per tile.
  *
  * Both products are issued transposed so that a query is a COLUMN of every
  * accumulator: S^T = K Q^T (A = K tile from LDS, B = Q^T held in registers)
@@ -29,10 +29,17 @@
  *
  * LDS layout: K tile row-major [64][128+8] bf16 (272 B rows = 16 B x odd, so
  * the 16 consecutive keys a ds_read_b128 phase touches fall in distinct
- * banks). V tile transposed [128][64+8] with the 16 keys of every MFMA
- * k-step stored in the order the P^T registers hold them
- * (pos = 8*((key/4)&1) + 4*((key/8)&1) + key%4), which makes every A operand
- * of the second product a single ds_read_b128.
+ * banks). V tile row-major too, [64][128+32] (320 B rows); the V^T operand
+ * is produced by the LDS transpose read ds_read_b64_tr_b16, which hands lane
+ * i of a 16-lane group column i of a 4-row x 16-column block: four
+ * consecutive keys of one head dim, which is exactly the group of keys that
+ * four consecutive P^T registers of that lane belong to. With 320 B rows the
+ * four rows of a group fall in disjoint banks.
+ *
+ * The running max is only raised when some query of the wave exceeds it by
+ * more than 2^8 (the accumulators are then rescaled); otherwise the
+ * exponentials are taken against the older max. Softmax is invariant to that
+ * shift, and exp2 arguments stay <= 8, far from overflow.
  *
  * Workgroups are numbered so that each XCD (own L2) walks a contiguous range
  * of (head, query-tile) pairs: the K/V of a head are then fetched into one
@@ -45,6 +52,8 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
@@ -54,18 +63,29 @@ constexpr int BM = 128;            /* queries per workgroup (32 per wave) */
 constexpr int BN = 64;             /* keys per tile */
 constexpr int HD = 128;
 constexpr int THREADS = 256;
-constexpr int KS = HD + 8;         /* K tile row stride in elements */
-constexpr int VS = BN + 8;         /* V^T tile row stride in elements */
+constexpr int KS = HD + 8;         /* K tile row stride in elements (272 B) */
+constexpr int VS = HD + 32;        /* V tile row stride in elements (320 B) */
+constexpr int K_TILE = BN * KS;    /* elements */
+constexpr int V_TILE = BN * VS;
+constexpr int STAGE = K_TILE + V_TILE;
 constexpr int XCDS = 8;
+constexpr float RESCALE_THRESHOLD = 8.0f;   /* log2 units */
 
-struct TileRegs {
-    uint4 k[4];
-    uint4 v[4];
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+struct TileRegs {          /* this thread's share of one K/V tile: 8 x 16 B */
+    u32x4 k0, k1, k2, k3, v0, v1, v2, v3;
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     f32x2 p = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2));
+}
+
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float d;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
 }
 
 /* Max (or sum) of a value with the same lane of the other half-wave. */
@@ -78,50 +98,44 @@ __device__ __forceinline__ float half_swap_sum(float v) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-/* HBM -> registers: this thread's share of the 64-key tile starting at k0.
- * K: 16 B pieces in row order. V: four consecutive keys x eight dims, so the
- * 4x8 block can be transposed in registers. Rows past seq_k read as zero. */
-__device__ __forceinline__ void fetch_tile(TileRegs &t, const uint16_t *kbase, const uint16_t *vbase,
-                                           int ldi, int k0, int seq_k, int tid) {
-    const int krow = tid >> 4, kcol = (tid & 15) * 8;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int vkey = 4 * (lane & 15), vcol = (4 * wave + (lane >> 4)) * 8;
-#pragma unroll
-    for (int c = 0; c < 4; c++) {
-        int kk = k0 + krow + 16 * c;
-        t.k[c] = kk < seq_k ? *reinterpret_cast<const uint4 *>(kbase + (size_t)kk * ldi + kcol)
-                            : make_uint4(0, 0, 0, 0);
-        int vk = k0 + vkey + c;
-        t.v[c] = vk < seq_k ? *reinterpret_cast<const uint4 *>(vbase + (size_t)vk * ldi + vcol)
-                            : make_uint4(0, 0, 0, 0);
-    }
+/* HBM -> registers: 16 B pieces of the 64-key tile whose first row is at
+ * `kt` / `vt` (wave-uniform pointers), at this thread's four row offsets. */
+__device__ __forceinline__ void fetch_tile(TileRegs &t, const uint16_t *kt, const uint16_t *vt,
+                                           const uint32_t *off) {
+    const char *kc = reinterpret_cast<const char *>(kt), *vc = reinterpret_cast<const char *>(vt);
+    t.k0 = *reinterpret_cast<const u32x4 *>(kc + off[0]);
+    t.v0 = *reinterpret_cast<const u32x4 *>(vc + off[0]);
+    t.k1 = *reinterpret_cast<const u32x4 *>(kc + off[1]);
+    t.v1 = *reinterpret_cast<const u32x4 *>(vc + off[1]);
+    t.k2 = *reinterpret_cast<const u32x4 *>(kc + off[2]);
+    t.v2 = *reinterpret_cast<const u32x4 *>(vc + off[2]);
+    t.k3 = *reinterpret_cast<const u32x4 *>(kc + off[3]);
+    t.v3 = *reinterpret_cast<const u32x4 *>(vc + off[3]);
 }
 
-/* Registers -> LDS. */
-__device__ __forceinline__ void store_tile(const TileRegs &t, uint16_t *Ks, uint16_t *Vt, int tid) {
-    const int krow = tid >> 4, kcol = (tid & 15) * 8;
-#pragma unroll
-    for (int c = 0; c < 4; c++)
-        *reinterpret_cast<uint4 *>(&Ks[(krow + 16 * c) * KS + kcol]) = t.k[c];
+/* Registers -> LDS stage. */
+__device__ __forceinline__ void store_tile(const TileRegs &t, uint16_t *stage, int tid) {
+    const int row = tid >> 4, col = (tid & 15) * 8;
+    uint16_t *kp = &stage[row * KS + col], *vp = &stage[K_TILE + row * VS + col];
+    *reinterpret_cast<u32x4 *>(kp) = t.k0;
+    *reinterpret_cast<u32x4 *>(vp) = t.v0;
+    *reinterpret_cast<u32x4 *>(kp + 16 * KS) = t.k1;
+    *reinterpret_cast<u32x4 *>(vp + 16 * VS) = t.v1;
+    *reinterpret_cast<u32x4 *>(kp + 32 * KS) = t.k2;
+    *reinterpret_cast<u32x4 *>(vp + 32 * VS) = t.v2;
+    *reinterpret_cast<u32x4 *>(kp + 48 * KS) = t.k3;
+    *reinterpret_cast<u32x4 *>(vp + 48 * VS) = t.v3;
+}
 
-    const int lane = tid & 63, wave = tid >> 6;
-    const int m = lane & 15;                       /* group of 4 keys */
-    const int d0 = (4 * wave + (lane >> 4)) * 8;
-    /* position of key 4m inside its 16-key k-step, in P^T register order */
-    const int pos = 16 * (m >> 2) + 8 * (m & 1) + 4 * ((m >> 1) & 1);
-    const uint32_t a0[4] = {t.v[0].x, t.v[0].y, t.v[0].z, t.v[0].w};
-    const uint32_t a1[4] = {t.v[1].x, t.v[1].y, t.v[1].z, t.v[1].w};
-    const uint32_t a2[4] = {t.v[2].x, t.v[2].y, t.v[2].z, t.v[2].w};
-    const uint32_t a3[4] = {t.v[3].x, t.v[3].y, t.v[3].z, t.v[3].w};
+/* Byte offsets of this thread's four rows of a tile starting at key k0; rows
+ * past the end are redirected to the last valid row (their scores are masked
+ * and their probabilities are exactly zero, so the values never matter). */
+__device__ __forceinline__ void tile_offsets(uint32_t (&off)[4], int tid, int ldi, int k0, int seq_k) {
+    const int row = tid >> 4, col = (tid & 15) * 8;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        uint2 even, odd;
-        even.x = __builtin_amdgcn_perm(a1[i], a0[i], 0x05040100u);
-        even.y = __builtin_amdgcn_perm(a3[i], a2[i], 0x05040100u);
-        odd.x = __builtin_amdgcn_perm(a1[i], a0[i], 0x07060302u);
-        odd.y = __builtin_amdgcn_perm(a3[i], a2[i], 0x07060302u);
-        *reinterpret_cast<uint2 *>(&Vt[(d0 + 2 * i) * VS + pos]) = even;
-        *reinterpret_cast<uint2 *>(&Vt[(d0 + 2 * i + 1) * VS + pos]) = odd;
+    for (int c = 0; c < 4; c++) {
+        int r = min(row + 16 * c, seq_k - 1 - k0);
+        off[c] = (uint32_t)(r * ldi + col) * 2u;
     }
 }
 
@@ -131,8 +145,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
                int seq_q, int seq_k, int q_tiles, int total_work, int work_per_xcd,
                int kv_group, float scale_log2, const int *__restrict__ key_mask) {
-    __shared__ __align__(16) uint16_t Ks[BN * KS];
-    __shared__ __align__(16) uint16_t Vt[HD * VS];
+    extern __shared__ __align__(16) uint16_t lds[];     /* two stages of [K tile | V tile] */
 
     /* XCD-aware numbering: hardware deals workgroups round-robin to the 8
      * XCDs, so id%8 is the XCD; give each XCD a contiguous slice of the
@@ -154,12 +167,9 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     /* Q^T as B operands: lane (query col, half hh) holds dims 16t + 8hh .. +7. */
     bf16x8 qb[8];
     {
-        const uint16_t *qp = q + (size_t)qrow * ldi + (size_t)head * HD + 8 * hh;
+        const uint16_t *qp = q + (size_t)min(qrow, seq_q - 1) * ldi + (size_t)head * HD + 8 * hh;
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
-            uint4 raw = qrow < seq_q ? *reinterpret_cast<const uint4 *>(qp + 16 * t) : make_uint4(0, 0, 0, 0);
-            qb[t] = __builtin_bit_cast(bf16x8, raw);
-        }
+        for (int t = 0; t < 8; t++) qb[t] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 16 * t));
     }
 
     f32x16 o[4];
@@ -173,26 +183,73 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     if (CAUSAL) k_end = min(seq_k, q0 + BM);       /* keys beyond the last query of the block are never valid */
     const int ntiles = (k_end + BN - 1) / BN;
 
+    /* LDS read addresses (elements, relative to a stage).
+     * K operand: row = key (col [+32]), 16 B at dims 16t + 8hh.
+     * V^T operand: transpose read; lane supplies row 4hh + (lane%16)/4 (+16t, +8)
+     * and columns 16*((lane/16)%2) + 4*(lane%4) (+32db). */
+    const int k_rd = col * KS + 8 * hh;
+    const int v_rd = K_TILE + (4 * hh + ((lane & 15) >> 2)) * VS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+    /* Row offsets of this thread's 16 B pieces: one set for full tiles, one for
+     * the last tile (rows past seq_k redirected to the last valid row). */
+    const int last_k0 = (ntiles - 1) * BN;
+    uint32_t off_full[4], off_last[4];
+    tile_offsets(off_full, tid, ldi, 0, BN);
+    tile_offsets(off_last, tid, ldi, last_k0, seq_k);
+
+    /* ---- prologue: tile 0 -> stage 0, tile 1 -> registers. Tile indices past
+     * the end are clamped to the last tile: the copy is redundant but keeps the
+     * pipeline free of control flow. ---- */
     TileRegs tile;
-    if (ntiles > 0) fetch_tile(tile, kbase, vbase, ldi, 0, seq_k, tid);
+    {
+        uint32_t off[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) off[c] = ntiles > 1 ? off_full[c] : off_last[c];
+        fetch_tile(tile, kbase, vbase, off);
+        store_tile(tile, lds, tid);
+        const int kn = min(BN, last_k0);
+#pragma unroll
+        for (int c = 0; c < 4; c++) off[c] = kn == last_k0 ? off_last[c] : off_full[c];
+        fetch_tile(tile, kbase + (size_t)kn * ldi, vbase + (size_t)kn * ldi, off);
+    }
+    __syncthreads();
 
     for (int it = 0; it < ntiles; it++) {
         const int k0 = it * BN;
-        __syncthreads();                           /* everyone is done reading the previous tile */
-        store_tile(tile, Ks, Vt, tid);
-        __syncthreads();
-        if (it + 1 < ntiles) fetch_tile(tile, kbase, vbase, ldi, k0 + BN, seq_k, tid);
+        uint16_t *cur = lds + (it & 1) * STAGE;
 
-        /* ---- S^T = K Q^T : two 32-key blocks, 8 k-steps over the head dim ---- */
+        /* tile it+1: registers -> the other stage (its last readers passed the barrier
+         * that ended the previous iteration); tile it+2: HBM -> registers */
+        store_tile(tile, lds + ((it + 1) & 1) * STAGE, tid);
+        {
+            const int kn = min(k0 + 2 * BN, last_k0);
+            const bool is_last = kn == last_k0;
+            uint32_t off[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) off[c] = is_last ? off_last[c] : off_full[c];
+            fetch_tile(tile, kbase + (size_t)kn * ldi, vbase + (size_t)kn * ldi, off);
+        }
+
+        /* ---- S^T = K Q^T : two 32-key blocks, 8 k-steps over the head dim.
+         * All 16 A operands are requested from LDS up front so their latency
+         * overlaps instead of gating every MFMA. ---- */
         f32x16 s0, s1;
+        {
+            u32x4 ka[8], kb[8];
 #pragma unroll
-        for (int r = 0; r < 16; r++) { s0[r] = 0.0f; s1[r] = 0.0f; }
+            for (int t = 0; t < 8; t++) {
+                ka[t] = *reinterpret_cast<const u32x4 *>(&cur[k_rd + 16 * t]);
+                kb[t] = *reinterpret_cast<const u32x4 *>(&cur[k_rd + 32 * KS + 16 * t]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[0]), qb[0], zero, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kb[0]), qb[0], zero, 0, 0, 0);
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
-            bf16x8 ka = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(&Ks[col * KS + 16 * t + 8 * hh]));
-            bf16x8 kb = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(&Ks[(32 + col) * KS + 16 * t + 8 * hh]));
-            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qb[t], s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kb, qb[t], s1, 0, 0, 0);
+            for (int t = 1; t < 8; t++) {
+                s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[t]), qb[t], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kb[t]), qb[t], s1, 0, 0, 0);
+            }
         }
         /* register r of block b holds key k0 + 32b + 8(r/4) + 4hh + r%4 for query qrow */
 
@@ -214,24 +271,34 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             const int lim = qrow - k0 - 4 * hh;    /* key offset const_r valid iff const_r <= lim */
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int off = 8 * (r >> 2) + (r & 3);
-                if (off > lim) s0[r] = -INFINITY;
-                if (off + 32 > lim) s1[r] = -INFINITY;
+                const int koff = 8 * (r >> 2) + (r & 3);
+                if (koff > lim) s0[r] = -INFINITY;
+                if (koff + 32 > lim) s1[r] = -INFINITY;
             }
         }
 
         /* ---- online softmax, one query per lane ---- */
-        float mx = fmaxf(s0[0], s1[0]);
+        float mx = max3(s0[0], s0[1], s1[0]);
+        mx = max3(mx, s1[1], s0[2]);
 #pragma unroll
-        for (int r = 1; r < 16; r++) mx = fmaxf(mx, fmaxf(s0[r], s1[r]));
-        mx = half_swap_max(mx);
-        const float m_new = fmaxf(m_run, mx * scale_log2);
-        const float m_ref = m_new == -INFINITY ? 0.0f : m_new;   /* finite while every key so far is masked */
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
-        m_run = m_new;
-        const float neg_m = -m_ref;
+        for (int r = 3; r < 16; r += 2) mx = max3(mx, s0[r], s0[r + 1 < 16 ? r + 1 : r]);
+#pragma unroll
+        for (int r = 2; r < 16; r += 2) mx = max3(mx, s1[r], s1[r + 1]);
+        mx = half_swap_max(mx) * scale_log2;
 
-        float psum = 0.0f;
+        if (__any(mx > m_run + RESCALE_THRESHOLD)) {
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - (m_new == -INFINITY ? 0.0f : m_new));
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < 4; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+        }
+        const float neg_m = m_run == -INFINITY ? 0.0f : -m_run;   /* finite while every key so far is masked */
+
+        float psum0 = 0.0f, psum1 = 0.0f;
         uint32_t pw[16];                            /* P^T as bf16 pairs: pw[4*t + j] = k-step t, elements 2j, 2j+1 */
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
@@ -239,30 +306,40 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             float p1 = __builtin_amdgcn_exp2f(fmaf(s0[r + 1], scale_log2, neg_m));
             float p2 = __builtin_amdgcn_exp2f(fmaf(s1[r], scale_log2, neg_m));
             float p3 = __builtin_amdgcn_exp2f(fmaf(s1[r + 1], scale_log2, neg_m));
-            psum += (p0 + p1) + (p2 + p3);
+            psum0 += p0 + p1;
+            psum1 += p2 + p3;
             pw[r >> 1] = pack_bf16(p0, p1);
             pw[8 + (r >> 1)] = pack_bf16(p2, p3);
         }
-        l_run = fmaf(l_run, alpha, psum);           /* per half-wave partial; halves are added at the end */
+        l_run += psum0 + psum1;                     /* per half-wave partial; halves are added at the end */
 
-        if (__any(alpha != 1.0f)) {
+        /* ---- O^T += V^T P^T : 4 k-steps of 16 keys x 4 dim blocks; the V^T
+         * operands of two k-steps are requested together ---- */
 #pragma unroll
-            for (int db = 0; db < 4; db++)
+        for (int tp = 0; tp < 4; tp += 2) {
+            s16x4 lo[2][4], hi[2][4];
 #pragma unroll
-                for (int r = 0; r < 16; r++) o[db][r] *= alpha;
-        }
-
-        /* ---- O^T += V^T P^T : 4 dim blocks x 4 k-steps of 16 keys ---- */
+            for (int u = 0; u < 2; u++)
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            uint4 praw = make_uint4(pw[4 * t], pw[4 * t + 1], pw[4 * t + 2], pw[4 * t + 3]);
-            bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
+                for (int db = 0; db < 4; db++) {
+                    const uint16_t *vp = &cur[v_rd + 16 * (tp + u) * VS + 32 * db];
+                    lo[u][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp));
+                    hi[u][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 8 * VS));
+                }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int db = 0; db < 4; db++) {
-                bf16x8 va = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(&Vt[(32 * db + col) * VS + 16 * t + 8 * hh]));
-                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, o[db], 0, 0, 0);
+            for (int u = 0; u < 2; u++) {
+                const int t = tp + u;
+                uint4 praw = make_uint4(pw[4 * t], pw[4 * t + 1], pw[4 * t + 2], pw[4 * t + 3]);
+                bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
+#pragma unroll
+                for (int db = 0; db < 4; db++) {
+                    s16x8 both = __builtin_shufflevector(lo[u][db], hi[u][db], 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pb, o[db], 0, 0, 0);
+                }
             }
         }
+        __syncthreads();
     }
 
     /* ---- normalise and store: lane holds dims 32db + 8g + 4hh + {0..3} of query qrow ---- */
@@ -282,6 +359,24 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     }
 }
 
+constexpr size_t LDS_BYTES = 2 * STAGE * sizeof(uint16_t);
+
+template <bool C, bool M>
+int launch(hipStream_t st, dim3 grid, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
+           const uint16_t *v, int ldi, int seq_q, int seq_k, int q_tiles, int total, int per_xcd,
+           int kv_group, float scale_log2, const int *key_mask) {
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd128<C, M>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        configured = true;
+    }
+    hipLaunchKernelGGL((k_fa_fwd_hd128<C, M>), grid, dim3(THREADS), LDS_BYTES, st, out, ldo, q, k, v, ldi,
+                       seq_q, seq_k, q_tiles, total, per_xcd, kv_group, scale_log2, key_mask);
+    return (int)hipGetLastError();
+}
+
 }  // namespace
 
 extern "C" int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uint16_t *q,
@@ -291,18 +386,14 @@ extern "C" int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uin
     const int q_tiles = (seq_q + BM - 1) / BM;
     const int total = q_tiles * heads;
     const int per_xcd = (total + XCDS - 1) / XCDS;
-    const dim3 grid(per_xcd * XCDS), block(THREADS);
+    const dim3 grid(per_xcd * XCDS);
     const float scale_log2 = scale * 1.4426950408889634f;
     const int kv_group = heads / kv_heads;
     hipStream_t st = (hipStream_t)stream;
-#define FA_LAUNCH(C, M)                                                                          \
-    hipLaunchKernelGGL((k_fa_fwd_hd128<C, M>), grid, block, 0, st, out, ldo, q, k, v, ldi, seq_q, \
-                       seq_k, q_tiles, total, per_xcd, kv_group, scale_log2, key_mask)
     if (causal) {
-        if (key_mask) FA_LAUNCH(true, true); else FA_LAUNCH(true, false);
-    } else {
-        if (key_mask) FA_LAUNCH(false, true); else FA_LAUNCH(false, false);
+        if (key_mask) return launch<true, true>(st, grid, out, ldo, q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, kv_group, scale_log2, key_mask);
+        return launch<true, false>(st, grid, out, ldo, q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, kv_group, scale_log2, key_mask);
     }
-#undef FA_LAUNCH
-    return (int)hipGetLastError();
+    if (key_mask) return launch<false, true>(st, grid, out, ldo, q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, kv_group, scale_log2, key_mask);
+    return launch<false, false>(st, grid, out, ldo, q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, kv_group, scale_log2, key_mask);
 }

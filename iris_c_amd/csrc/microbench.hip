@@ -1,0 +1,117 @@
+/*
+ * Machine-ceiling microbenchmarks reported next to the kernel numbers:
+ * what this GPU sustains for back-to-back bf16 MFMA, for a plain HBM copy,
+ * for 128-bit LDS reads and for v_exp_f32. Bench infrastructure, built into
+ * its own library (libiris_microbench.so); the product library does not
+ * contain it.
+ */
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+/* 4 independent accumulator chains per wave, `iters` x 4 MFMAs each. */
+__global__ void __launch_bounds__(256) k_mfma_peak(float *sink, int iters) {
+    f32x16 acc[4];
+    for (int a = 0; a < 4; a++)
+        for (int r = 0; r < 16; r++) acc[a][r] = 0.0f;
+    uint4 raw = make_uint4(0x3f803f80u + threadIdx.x, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
+    bf16x8 x = __builtin_bit_cast(bf16x8, raw), y = x;
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int a = 0; a < 4; a++) acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x, y, acc[a], 0, 0, 0);
+    }
+    float s = 0.0f;
+    for (int a = 0; a < 4; a++)
+        for (int r = 0; r < 16; r++) s += acc[a][r];
+    if (s == 12345.678f) sink[0] = s;
+}
+
+__global__ void __launch_bounds__(256) k_copy(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 * 4 + threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        size_t j = i + (size_t)u * 256;
+        if (j < n) dst[j] = src[j];
+    }
+}
+
+/* In-place read-modify-write of the same buffer (the norm+rope access pattern). */
+__global__ void __launch_bounds__(256) k_rmw(uint4 *__restrict__ buf, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 * 4 + threadIdx.x;
+    uint4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        size_t j = i + (size_t)u * 256;
+        v[u] = j < n ? buf[j] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        size_t j = i + (size_t)u * 256;
+        v[u].x ^= 1u;
+        if (j < n) buf[j] = v[u];
+    }
+}
+
+/* Every wave reads 16 B per lane from a padded row layout (row stride 272 B),
+ * the access pattern of an MFMA A operand; `iters` x 8 reads. */
+__global__ void __launch_bounds__(256) k_lds_read(float *sink, int iters) {
+    __shared__ __align__(16) uint16_t lds[64 * 136];
+    for (int i = threadIdx.x; i < 64 * 136; i += 256) lds[i] = (uint16_t)i;
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const uint16_t *p = &lds[(lane & 31) * 136 + 8 * (lane >> 5)];
+    uint4 acc = make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            u32x4 v = *reinterpret_cast<const volatile u32x4 *>(p + 16 * t + ((i & 1) ? 32 * 136 : 0));
+            acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w;
+        }
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) sink[0] = 1.0f;
+}
+
+__global__ void __launch_bounds__(256) k_exp(float *sink, int iters) {
+    float v[8];
+    for (int j = 0; j < 8; j++) v[j] = -1.0f - threadIdx.x * 1e-3f - j;
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = __builtin_amdgcn_exp2f(v[j]) - 2.0f;
+    }
+    float s = 0.0f;
+    for (int j = 0; j < 8; j++) s += v[j];
+    if (s == 12345.678f) sink[0] = s;
+}
+
+}  // namespace
+
+extern "C" {
+int iris_mb_mfma(void *stream, float *sink, int blocks, int iters) {
+    hipLaunchKernelGGL(k_mfma_peak, dim3(blocks), dim3(256), 0, (hipStream_t)stream, sink, iters);
+    return (int)hipGetLastError();
+}
+int iris_mb_copy(void *stream, void *dst, const void *src, size_t bytes) {
+    size_t n = bytes / 16;
+    hipLaunchKernelGGL(k_copy, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream,
+                       (uint4 *)dst, (const uint4 *)src, n);
+    return (int)hipGetLastError();
+}
+int iris_mb_rmw(void *stream, void *buf, size_t bytes) {
+    size_t n = bytes / 16;
+    hipLaunchKernelGGL(k_rmw, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream, (uint4 *)buf, n);
+    return (int)hipGetLastError();
+}
+int iris_mb_lds(void *stream, float *sink, int blocks, int iters) {
+    hipLaunchKernelGGL(k_lds_read, dim3(blocks), dim3(256), 0, (hipStream_t)stream, sink, iters);
+    return (int)hipGetLastError();
+}
+int iris_mb_exp(void *stream, float *sink, int blocks, int iters) {
+    hipLaunchKernelGGL(k_exp, dim3(blocks), dim3(256), 0, (hipStream_t)stream, sink, iters);
+    return (int)hipGetLastError();
+}
+}
