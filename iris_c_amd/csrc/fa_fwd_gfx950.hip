@@ -77,6 +77,13 @@ struct TileRegs {          /* this thread's share of one K/V tile: 8 x 16 B */
     u32x4 k0, k1, k2, k3, v0, v1, v2, v3;
 };
 
+/* Workgroup barrier that only waits for this wave's LDS traffic. __syncthreads()
+ * would also wait for outstanding global loads (vmcnt(0)), i.e. for the tile
+ * that was requested precisely so that it arrives later. */
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     f32x2 p = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2));
@@ -242,6 +249,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                 kb[t] = *reinterpret_cast<const u32x4 *>(&cur[k_rd + 32 * KS + 16 * t]);
             }
             __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(1);
             const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
             s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[0]), qb[0], zero, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kb[0]), qb[0], zero, 0, 0, 0);
@@ -250,6 +258,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                 s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[t]), qb[t], s0, 0, 0, 0);
                 s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kb[t]), qb[t], s1, 0, 0, 0);
             }
+            __builtin_amdgcn_s_setprio(0);
         }
         /* register r of block b holds key k0 + 32b + 8(r/4) + 4hh + r%4 for query qrow */
 
@@ -327,6 +336,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                     hi[u][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 8 * VS));
                 }
             __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int u = 0; u < 2; u++) {
                 const int t = tp + u;
@@ -338,8 +348,9 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                     o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pb, o[db], 0, 0, 0);
                 }
             }
+            __builtin_amdgcn_s_setprio(0);
         }
-        __syncthreads();
+        lds_barrier();
     }
 
     /* ---- normalise and store: lane holds dims 32db + 8g + 4hh + {0..3} of query qrow ---- */

@@ -15,6 +15,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "iris_dev.h"

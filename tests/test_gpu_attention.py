@@ -16,6 +16,12 @@ def dev():
     return Dev()
 
 
+@pytest.fixture
+def fa():
+    """Name of the matrix-core kernel every head_dim-128, aligned call must take."""
+    return "fa_hd128"
+
+
 def gpu_attention(dev, case, **over):
     a = dict(case); a.update(over)
     out, kernel = dev.attention(a["buf"], a["ldi"], 0, a["q_dim"], a["q_dim"] + a["kv_dim"], a["seq"], a["seq"],
@@ -44,10 +50,10 @@ def after_norm_rope(dev, case):
 
 
 # ------------------------------------------------------------------ the five configurations, shrunk
-def test_c1_plumbing_full_size(dev, orc):
+def test_c1_plumbing_full_size(dev, orc, fa):
     case = after_norm_rope(dev, W.c1())           # 64 text + 16x16 image, 24 heads
     got, kernel = gpu_attention(dev, case)
-    assert kernel == "fa_hd128"
+    assert kernel == fa
     assert_close(got, cpu_attention(orc, case), "C1")
     # and against the reference-shaped f32 flash attention on the same inputs
     f = O.bf16_to_f32(case["buf"])
@@ -56,26 +62,26 @@ def test_c1_plumbing_full_size(dev, orc):
 
 
 @pytest.mark.parametrize("maker,shrink", [(W.c2, 8), (W.c5, 32)])
-def test_joint_attention_shrunk(dev, orc, maker, shrink):
+def test_joint_attention_shrunk(dev, orc, fa, maker, shrink):
     case = after_norm_rope(dev, maker(shrink))
     got, kernel = gpu_attention(dev, case)
-    assert kernel == "fa_hd128"
+    assert kernel == fa
     assert_close(got, cpu_attention(orc, case), case["name"])
 
 
-def test_c3_cfg_pair_with_key_mask(dev, orc):
+def test_c3_cfg_pair_with_key_mask(dev, orc, fa):
     for case in W.c3(shrink=8):
         case = after_norm_rope(dev, case)
         got, kernel = gpu_attention(dev, case)
-        assert kernel == "fa_hd128"
+        assert kernel == fa
         assert_close(got, cpu_attention(orc, case), case["name"])
 
 
 @pytest.mark.parametrize("shrink", [1, 4])
-def test_c4_causal_gqa_padding(dev, orc, shrink):
+def test_c4_causal_gqa_padding(dev, orc, fa, shrink):
     case = after_norm_rope(dev, W.c4(shrink))
     got, kernel = gpu_attention(dev, case)
-    assert kernel == "fa_hd128"
+    assert kernel == fa
     assert_close(got, cpu_attention(orc, case), "C4")
 
 
@@ -114,10 +120,11 @@ def test_c5_full_size_sampled_rows(dev, orc):
     assert_close(got[rows], cpu_attention(orc, case, rows=rows), "C5 sampled")
 
 
-def test_c3_full_size_masked_equals_compacted(dev, orc):
+def test_c3_full_size_masked_equals_compacted(dev, orc, fa):
     cond, unc = W.c3()
     unc = after_norm_rope(dev, unc)
-    got, _ = gpu_attention(dev, unc)
+    got, kernel = gpu_attention(dev, unc)
+    assert kernel == fa
     rows = sample_rows(unc["seq"], n=20)
     assert_close(got[rows], cpu_attention(orc, unc, rows=rows), "C3 uncond sampled")
     # masked keys == the same problem with those K/V rows removed
@@ -138,17 +145,17 @@ def random_case(seed, seq_q, seq_k, heads, kv_heads, hd=128, pad=0, sigma=1.0):
 
 @pytest.mark.parametrize("seq_q,seq_k", [(1, 1), (1, 64), (5, 63), (33, 65), (128, 128), (129, 191), (200, 31), (257, 1000)])
 @pytest.mark.parametrize("causal", [False, True])
-def test_ragged_shapes(dev, orc, seq_q, seq_k, causal):
+def test_ragged_shapes(dev, orc, fa, seq_q, seq_k, causal):
     heads, kv = 4, 2
     buf, ldi = random_case(seq_q * 7 + seq_k, seq_q, seq_k, heads, kv)
     qd, kd = heads * 128, kv * 128
     out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, 128, 0.0884, causal)
-    assert kernel == "fa_hd128"
+    assert kernel == fa
     want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, 128, 0.0884, causal)
     assert_close(O.bf16_to_f32(out[:seq_q]), want, f"{seq_q}x{seq_k} causal={causal}")
 
 
-def test_random_key_masks_and_empty_rows(dev, orc):
+def test_random_key_masks_and_empty_rows(dev, orc, fa):
     heads, seq = 3, 300
     buf, ldi = random_case(5, seq, seq, heads, heads)
     rng = np.random.default_rng(6)
@@ -168,7 +175,7 @@ def test_random_key_masks_and_empty_rows(dev, orc):
     assert np.all(O.bf16_to_f32(out) == 0.0)
 
 
-def test_large_scores_stay_finite(dev, orc):
+def test_large_scores_stay_finite(dev, orc, fa):
     heads, seq = 2, 130
     buf, ldi = random_case(9, seq, seq, heads, heads, sigma=6.0)     # |score| up to ~100
     out, _ = dev.attention(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, 0.0884)
@@ -179,12 +186,12 @@ def test_large_scores_stay_finite(dev, orc):
     assert mx <= 0.13 and mean <= 4e-3      # outputs are O(6): same relative bar as 2e-2 on O(1) values
 
 
-def test_output_stride_and_interior_pointers(dev, orc):
+def test_output_stride_and_interior_pointers(dev, orc, fa):
     heads, seq = 2, 70
     buf, ldi = random_case(11, seq, seq, heads, heads, pad=64)
     ldo, out_col = 2 * 256 + 8, 256
     out, kernel = dev.attention(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, 0.0884, ldo=ldo, out_col=out_col)
-    assert kernel == "fa_hd128"
+    assert kernel == fa
     want = orc.attention_bf16(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, 0.0884)
     assert_close(O.bf16_to_f32(out[:, out_col:out_col + 256]), want, "strided out")
     assert np.all(out[:, :out_col] == 0x7fc0) and np.all(out[:, out_col + 256:] == 0x7fc0)
