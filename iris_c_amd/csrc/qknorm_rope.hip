@@ -25,11 +25,14 @@
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kUnroll = 4;                       /* vectors in flight per 16-lane row */
+/* Measured on C2 (cold rows): 2 -> 13.2 us, 1 -> 14.1, 4 -> 14.0, 8 -> 16.3; nontemporal
+ * loads/stores gain nothing cold and cost 30% when the rows sit in the Infinity Cache. */
+constexpr int kUnroll = 2;                       /* vectors in flight per 16-lane row */
 constexpr int kUnitsPerBlock = (kThreads / 16) * kUnroll;
 
 __device__ __forceinline__ float bf_lo(uint32_t u) { return __uint_as_float(u << 16); }
@@ -71,24 +74,46 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
     const int tcol = SPLIT ? 8 * (sub & 7) : 4 * sub;
     const float sgn = (SPLIT && sub < 8) ? -1.0f : 1.0f;
 
-    uint4 raw[kUnroll];
-    int tok[kUnroll];
+    /* Phase 1: request everything this thread needs for its kUnroll vectors --
+     * the 16 B of x and the matching cos/sin entries -- before touching any of
+     * it, so all the loads are in flight together. */
+    constexpr int TN = SPLIT ? 2 : 1;               /* float4 table loads per vector */
+    u32x4 raw[kUnroll];
+    float4 ct[kUnroll][TN], st[kUnroll][TN];
     uint16_t *ptr[kUnroll];
     bool isk[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
         int unit = first + u * (kThreads / 16);
-        bool live = unit < units;
+        const bool live = unit < units;
         unit = live ? unit : 0;
-        int s = (int)__umulhi((uint32_t)unit, magic);       /* unit / heads_total */
-        int h = unit - s * heads_total;
+        const int s = (int)__umulhi((uint32_t)unit, magic);       /* unit / heads_total */
+        const int h = unit - s * heads_total;
         isk[u] = h >= q_heads;
         uint16_t *base = isk[u] ? xk + (size_t)(h - q_heads) * 128 : xq + (size_t)h * 128;
         ptr[u] = live ? base + (size_t)s * ld + sub * 8 : nullptr;
-        tok[u] = s;
-        raw[u] = live ? *reinterpret_cast<const uint4 *>(ptr[u]) : make_uint4(0, 0, 0, 0);
+        raw[u] = live ? *reinterpret_cast<const u32x4 *>(ptr[u]) : u32x4{0, 0, 0, 0};
+        const float *cp = rope_cos + (size_t)s * 64 + tcol;
+        const float *sp = rope_sin + (size_t)s * 64 + tcol;
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+            ct[u][i] = *reinterpret_cast<const float4 *>(cp + 4 * i);
+            st[u][i] = *reinterpret_cast<const float4 *>(sp + 4 * i);
+        }
+    }
+    /* the norm weights of this lane's 8 dims (Q and, when present, K) */
+    float wq8[8], wk8[8];
+    {
+        const float4 a0 = *reinterpret_cast<const float4 *>(wq + sub * 8);
+        const float4 a1 = *reinterpret_cast<const float4 *>(wq + sub * 8 + 4);
+        const float *wks = heads_total > q_heads ? wk : wq;
+        const float4 b0 = *reinterpret_cast<const float4 *>(wks + sub * 8);
+        const float4 b1 = *reinterpret_cast<const float4 *>(wks + sub * 8 + 4);
+        wq8[0] = a0.x; wq8[1] = a0.y; wq8[2] = a0.z; wq8[3] = a0.w; wq8[4] = a1.x; wq8[5] = a1.y; wq8[6] = a1.z; wq8[7] = a1.w;
+        wk8[0] = b0.x; wk8[1] = b0.y; wk8[2] = b0.z; wk8[3] = b0.w; wk8[4] = b1.x; wk8[5] = b1.y; wk8[6] = b1.z; wk8[7] = b1.w;
     }
 
+    /* Phase 2: normalise, rotate, store. */
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
         if (!ptr[u]) continue;
@@ -99,24 +124,13 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
         for (int i = 0; i < 8; i++) ss = fmaf(e[i], e[i], ss);
         ss = row16_sum(ss);
         const float inv = 1.0f / sqrtf(ss * (1.0f / 128.0f) + eps);
-
-        const float *w = isk[u] ? wk : wq;
-        const float4 w0 = *reinterpret_cast<const float4 *>(w + sub * 8);
-        const float4 w1 = *reinterpret_cast<const float4 *>(w + sub * 8 + 4);
-        const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
 #pragma unroll
-        for (int i = 0; i < 8; i++) e[i] *= inv * wv[i];
+        for (int i = 0; i < 8; i++) e[i] *= inv * (isk[u] ? wk8[i] : wq8[i]);
 
-        const float *cp = rope_cos + (size_t)tok[u] * 64 + tcol;
-        const float *sp = rope_sin + (size_t)tok[u] * 64 + tcol;
         float o[8];
         if (SPLIT) {
-            const float4 c0 = *reinterpret_cast<const float4 *>(cp);
-            const float4 c1 = *reinterpret_cast<const float4 *>(cp + 4);
-            const float4 s0 = *reinterpret_cast<const float4 *>(sp);
-            const float4 s1 = *reinterpret_cast<const float4 *>(sp + 4);
-            const float cv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-            const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+            const float cv[8] = {ct[u][0].x, ct[u][0].y, ct[u][0].z, ct[u][0].w, ct[u][TN - 1].x, ct[u][TN - 1].y, ct[u][TN - 1].z, ct[u][TN - 1].w};
+            const float sv[8] = {st[u][0].x, st[u][0].y, st[u][0].z, st[u][0].w, st[u][TN - 1].x, st[u][TN - 1].y, st[u][TN - 1].z, st[u][TN - 1].w};
 #pragma unroll
             for (int i = 0; i < 8; i++) {
                 /* lanes 0-7 hold a (first half), lanes 8-15 hold b: a*c - b*s / b*c + a*s */
@@ -124,10 +138,8 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
                 o[i] = fmaf(sgn * other, sv[i], e[i] * cv[i]);
             }
         } else {
-            const float4 c = *reinterpret_cast<const float4 *>(cp);
-            const float4 s = *reinterpret_cast<const float4 *>(sp);
-            const float cv[4] = {c.x, c.y, c.z, c.w};
-            const float sv[4] = {s.x, s.y, s.z, s.w};
+            const float cv[4] = {ct[u][0].x, ct[u][0].y, ct[u][0].z, ct[u][0].w};
+            const float sv[4] = {st[u][0].x, st[u][0].y, st[u][0].z, st[u][0].w};
 #pragma unroll
             for (int p = 0; p < 4; p++) {
                 float a = e[2 * p], b = e[2 * p + 1];
@@ -135,12 +147,12 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
                 o[2 * p + 1] = fmaf(a, sv[p], b * cv[p]);
             }
         }
-        uint4 out;
+        u32x4 out;
         out.x = pack_bf16(o[0], o[1]);
         out.y = pack_bf16(o[2], o[3]);
         out.z = pack_bf16(o[4], o[5]);
         out.w = pack_bf16(o[6], o[7]);
-        *reinterpret_cast<uint4 *>(ptr[u]) = out;
+        *reinterpret_cast<u32x4 *>(ptr[u]) = out;
     }
 }
 
