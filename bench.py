@@ -29,6 +29,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 matrix peak (vendor figure)
 PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E peak
+# HBM bytes one C2 attention launch moves, from the FETCH_SIZE and WRITE_SIZE hardware counters scaled by a
+# 1 GiB copy kernel (profiles/k_fa_fwd_hd128__c2__hbm_traffic.txt): 103.7 MB read + 28.3 MB written.
+C2_ATTENTION_HBM_TRAFFIC = 132_046_000
 
 _vp = C.c_void_p
 
@@ -195,6 +198,52 @@ def per_launch_times(hip, stream, fn, reps):
     return [hip.elapsed_ms(a, b) for a, b in evs]
 
 
+# ----------------------------------------------------------------------------- machine ceilings
+def microbench_lib():
+    mb = C.CDLL(os.path.join(ROOT, "iris_c_amd", "libiris_microbench.so"))
+    mb.iris_mb_mfma.argtypes = [_vp, _vp, C.c_int, C.c_int]
+    mb.iris_mb_copy.argtypes = [_vp, _vp, _vp, C.c_size_t]
+    mb.iris_mb_rmw.argtypes = [_vp, _vp, C.c_size_t]
+    return mb
+
+
+def copy_only(dev, hip, stream, nbytes, reps):
+    """`reps` launches of the plain copy kernel (reads nbytes, writes nbytes)."""
+    lib, mb = dev.lib, microbench_lib()
+    src, dst = lib.iris_dev_alloc(nbytes), lib.iris_dev_alloc(nbytes)
+    assert src and dst
+    mb.iris_mb_copy(stream, dst, src, nbytes)
+    ms = event_time(hip, stream, lambda i: mb.iris_mb_copy(stream, dst, src, nbytes), reps)
+    dev.check()
+    lib.iris_dev_free(src); lib.iris_dev_free(dst)
+    return {"kernel": "k_copy", "bytes_read": nbytes, "bytes_written": nbytes, "launches": reps + 1,
+            "us_per_launch": round(ms * 1e3, 2), "gbps_read_plus_write": round(2 * nbytes / ms / 1e6, 1)}
+
+
+def machine_ceilings(dev, hip, stream):
+    """What this GPU sustains on the two limits the kernels are priced against: a loop of nothing but
+    v_mfma_f32_32x32x16_bf16 (4 waves x 1024 blocks), and a 16 B/lane copy / in-place update of 1 GiB."""
+    lib, mb = dev.lib, microbench_lib()
+    sink = lib.iris_dev_alloc(64)
+    blocks, iters = 1024, 4000
+    mb.iris_mb_mfma(stream, sink, blocks, 16)
+    ms = min(event_time(hip, stream, lambda i: mb.iris_mb_mfma(stream, sink, blocks, iters), 1) for _ in range(3))
+    mfma = blocks * 4 * iters * 4 * 32768 / ms / 1e9
+    n = 1 << 30
+    a, b = lib.iris_dev_alloc(n), lib.iris_dev_alloc(n)
+    assert a and b
+    mb.iris_mb_copy(stream, b, a, n)
+    cp = min(event_time(hip, stream, lambda i: mb.iris_mb_copy(stream, b, a, n), 2) for _ in range(3))
+    rw = min(event_time(hip, stream, lambda i: mb.iris_mb_rmw(stream, a, n), 2) for _ in range(3))
+    dev.check()
+    for p in (sink, a, b):
+        lib.iris_dev_free(p)
+    return {"mfma_only_tflops": round(mfma, 1), "mfma_only_frac_of_peak": round(mfma / PEAK_BF16_TFLOPS, 4),
+            "copy_1gib_gbps": round(2 * n / cp / 1e6, 1), "inplace_update_1gib_gbps": round(2 * n / rw / 1e6, 1),
+            "note": "measured ceilings of this GPU for a pure MFMA loop and for streaming 16 B per lane; "
+                    "bytes counted read + written"}
+
+
 # ----------------------------------------------------------------------------- CPU baseline
 def cpu_baseline(c):
     """The reference's BLAS-build CPU attention (heads over pthreads, per head
@@ -208,17 +257,21 @@ def cpu_baseline(c):
     cores = base.online_cpus()
     box_share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
     limit = min(cores, box_share) if box_share > 0 else cores
-    t0 = time.perf_counter()
-    _, threads = base.attention(q, k, v, c["heads"], c["kv_heads"], c["scale"], c["causal"], c["key_mask"],
-                                q_chunk=0, threads=limit)
-    dt = time.perf_counter() - t0
+    calls, times = 8, []                  # 8 full calls: a few seconds of wall clock, ~30 core-seconds
+    for _ in range(calls):
+        t0 = time.perf_counter()
+        _, threads = base.attention(q, k, v, c["heads"], c["kv_heads"], c["scale"], c["causal"], c["key_mask"],
+                                    q_chunk=0, threads=limit)
+        times.append(time.perf_counter() - t0)
+    dt = float(np.mean(times[1:]))        # first call pays page faults and thread start
     flops = attention_flops(c)
     x = np.ascontiguousarray(q.reshape(c["seq"], c["heads"], c["hd"]))
     t1 = time.perf_counter()
     base.norm_rope(x, c["wq"], c["cos"], c["sin"], c["eps"], c["split_half"])
     dn = time.perf_counter() - t1
     return {"value": round(flops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"one full {c['name']} attention call ({c['heads']}h x {c['seq']} tok, f32), {dt:.2f} s; "
+            "sample": f"{calls} full {c['name']} attention calls ({c['heads']}h x {c['seq']} tok, f32), mean of the last "
+                      f"{calls - 1}: {dt:.2f} s each; "
                       f"sgemm from {os.path.basename(base.provider)}; host has {cores} CPUs online",
             "attention_seconds": round(dt, 3),
             "norm_rope_gbps": round(2 * x.nbytes / dn / 1e9, 3), "norm_rope_cores": 1}
@@ -232,6 +285,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-configuration table")
+    ap.add_argument("--no-machine", action="store_true", help="skip the MFMA-only / stream-copy ceilings")
+    ap.add_argument("--copy-only", type=int, default=0, metavar="MiB",
+                    help="only launch the plain copy kernel on MiB of data, --steps times (the known-size "
+                         "launch that hardware byte counters are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (heads are independent, so the path would shard by "
@@ -242,6 +299,9 @@ def main():
     lib, hip = dev.lib, Hip()
     stream = lib.iris_dev_stream()
     rng = np.random.default_rng(20250101)
+    if args.copy_only:
+        print(json.dumps(copy_only(dev, hip, stream, args.copy_only << 20, args.steps)))
+        return
 
     c2 = make_config("C2", rng)
     copies = 8                             # 8 x 85 MB rows > 256 MB Infinity Cache: norm+rope reads come from HBM
@@ -280,7 +340,8 @@ def main():
                    "device": dev.name()},
         "roofline": {"kernel": "k_fa_fwd_hd128", "bound": "mfma", "achieved": round(flops / (att_ms * 1e-3) / 1e12, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / (att_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
-                     "traffic": None, "launch_ms": round(att_ms, 4), "launch_ms_min": round(float(np.min(att)), 4),
+                     "traffic": C2_ATTENTION_HBM_TRAFFIC, "traffic_unit": "bytes per launch (hardware counters, profiled separately)",
+                     "algorithmic_bytes": 4 * c2["seq"] * c2["q_dim"] * 2, "launch_ms": round(att_ms, 4), "launch_ms_min": round(float(np.min(att)), 4),
                      "flops_per_launch": flops},
         "norm_rope": {"kernel": "k_norm_rope_hd128", "bound": "hbm", "unit": "GB/s", "peak": PEAK_HBM_GBPS,
                       "bytes_per_call": q_bytes,
@@ -313,6 +374,19 @@ def main():
             r.free()
         out["shapes"] = shapes
 
+    if not args.no_machine:
+        out["machine"] = machine_ceilings(dev, hip, stream)
+        # The ABI takes device pointers, so `value` has no host transfer in it. For a caller that had the
+        # fused qkv rows in host memory, this is the rate with the upload of those rows counted.
+        row_bytes = c2["buf"].nbytes
+        d = lib.iris_dev_alloc(row_bytes)
+        lib.iris_dev_upload(d, c2["buf"].ctypes.data_as(_vp), row_bytes)
+        t0 = time.perf_counter()
+        lib.iris_dev_upload(d, c2["buf"].ctypes.data_as(_vp), row_bytes)
+        up = time.perf_counter() - t0
+        lib.iris_dev_free(d)
+        out["machine"]["host_upload_gbps"] = round(row_bytes / up / 1e9, 2)
+        out["machine"]["pcie_inclusive_tflops"] = round(flops / (up + ms_per_step * 1e-3) / 1e12, 2)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(c2)
     print(json.dumps(out))

@@ -56,8 +56,9 @@ int iris_dev_init(void) {
         return 0;
     }
     if (hipSetDevice(0) != hipSuccess) return 0;
-    snprintf(g_name, sizeof(g_name), "%s (%s, %d CUs)", prop.name, prop.gcnArchName,
-             prop.multiProcessorCount);
+    /* some hosts report an empty marketing name */
+    snprintf(g_name, sizeof(g_name), "%s (%s, %d CUs, %d MHz)", prop.name[0] ? prop.name : "AMD Instinct",
+             prop.gcnArchName, prop.multiProcessorCount, prop.clockRate / 1000);
     if (hipStreamCreate(&g_stream) != hipSuccess) return 0;
     g_ready = 1;
     g_last_error = 0;
