@@ -202,6 +202,7 @@ def per_launch_times(hip, stream, fn, reps):
 def microbench_lib():
     mb = C.CDLL(os.path.join(ROOT, "iris_c_amd", "libiris_microbench.so"))
     mb.iris_mb_mfma.argtypes = [_vp, _vp, C.c_int, C.c_int]
+    mb.iris_mb_mfma_data.argtypes = [_vp, _vp, _vp, C.c_int, C.c_int]
     mb.iris_mb_copy.argtypes = [_vp, _vp, _vp, C.c_size_t]
     mb.iris_mb_rmw.argtypes = [_vp, _vp, C.c_size_t]
     return mb
@@ -229,6 +230,12 @@ def machine_ceilings(dev, hip, stream):
     mb.iris_mb_mfma(stream, sink, blocks, 16)
     ms = min(event_time(hip, stream, lambda i: mb.iris_mb_mfma(stream, sink, blocks, iters), 1) for _ in range(3))
     mfma = blocks * 4 * iters * 4 * 32768 / ms / 1e9
+    # the same MFMA loop on N(0,1) bf16 operands, long enough (tens of ms) for the clock to settle
+    ops = dev.to_device(to_bf16(np.random.default_rng(7).standard_normal(8 * 256 * 8).astype(np.float32)))
+    it2 = 5000
+    mb.iris_mb_mfma_data(stream, ops, sink, blocks, 16)
+    ms2 = min(event_time(hip, stream, lambda i: mb.iris_mb_mfma_data(stream, ops, sink, blocks, it2), 1) for _ in range(3))
+    mfma_data = blocks * 4 * it2 * 16 * 32768 / ms2 / 1e9
     n = 1 << 30
     a, b = lib.iris_dev_alloc(n), lib.iris_dev_alloc(n)
     assert a and b
@@ -236,12 +243,15 @@ def machine_ceilings(dev, hip, stream):
     cp = min(event_time(hip, stream, lambda i: mb.iris_mb_copy(stream, b, a, n), 2) for _ in range(3))
     rw = min(event_time(hip, stream, lambda i: mb.iris_mb_rmw(stream, a, n), 2) for _ in range(3))
     dev.check()
-    for p in (sink, a, b):
+    for p in (sink, a, b, ops):
         lib.iris_dev_free(p)
     return {"mfma_only_tflops": round(mfma, 1), "mfma_only_frac_of_peak": round(mfma / PEAK_BF16_TFLOPS, 4),
+            "mfma_only_normal_data_tflops": round(mfma_data, 1),
+            "mfma_only_normal_data_frac_of_peak": round(mfma_data / PEAK_BF16_TFLOPS, 4),
             "copy_1gib_gbps": round(2 * n / cp / 1e6, 1), "inplace_update_1gib_gbps": round(2 * n / rw / 1e6, 1),
-            "note": "measured ceilings of this GPU for a pure MFMA loop and for streaming 16 B per lane; "
-                    "bytes counted read + written"}
+            "note": "measured ceilings of this GPU: a pure MFMA loop on constant operands (short burst) and on "
+                    "N(0,1) operands (sustained; the clock drops with the data-dependent power draw), and "
+                    "streaming 16 B per lane, bytes counted read + written"}
 
 
 # ----------------------------------------------------------------------------- CPU baseline

@@ -12,10 +12,13 @@
  *
  * Shape of the computation on CDNA4
  * ---------------------------------
- * One workgroup = 4 waves = 128 queries of one head; each wave owns 32
- * queries for the whole kernel. Keys/values stream through two LDS stages in
- * tiles of 64: while tile i is multiplied, tile i+1 moves registers -> LDS
- * and tile i+2 moves HBM -> registers; one barrier per tile.
+ * One workgroup = 8 waves = 256 queries of one head (4 waves = 128 queries
+ * when that would leave CUs without work); each wave owns 32 queries for the
+ * whole kernel, two waves share a SIMD. Keys/values stream through two LDS
+ * stages in tiles of 64: while tile i is multiplied, tile i+1 moves
+ * registers -> LDS and tile i+2 moves HBM -> registers; one barrier per tile.
+ * Every wave reads the whole K and V tile, so 256 queries per workgroup mean
+ * half the L2 -> LDS traffic and half the LDS writes per query of 128.
  *
  * Both products are issued transposed so that a query is a COLUMN of every
  * accumulator: S^T = K Q^T (A = K tile from LDS, B = Q^T held in registers)
@@ -59,10 +62,9 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 namespace {
 
-constexpr int BM = 128;            /* queries per workgroup (32 per wave) */
+/* A workgroup is WAVES (4 or 8) waves of 32 queries: BM = 32 * WAVES queries, 64 * WAVES threads. */
 constexpr int BN = 64;             /* keys per tile */
 constexpr int HD = 128;
-constexpr int THREADS = 256;
 constexpr int KS = HD + 8;         /* K tile row stride in elements (272 B) */
 constexpr int VS = HD + 32;        /* V tile row stride in elements (320 B) */
 constexpr int K_TILE = BN * KS;    /* elements */
@@ -73,8 +75,11 @@ constexpr float RESCALE_THRESHOLD = 8.0f;   /* log2 units */
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
-struct TileRegs {          /* this thread's share of one K/V tile: 8 x 16 B */
-    u32x4 k0, k1, k2, k3, v0, v1, v2, v3;
+/* This thread's share of one K/V tile: NP = 1024 / threads pieces of 16 B of K and of V,
+ * RSTEP = threads / 16 rows apart. */
+template <int NP>
+struct TileRegs {
+    u32x4 k[NP], v[NP];
 };
 
 /* Workgroup barrier that only waits for this wave's LDS traffic. __syncthreads()
@@ -107,52 +112,52 @@ __device__ __forceinline__ float half_swap_sum(float v) {
 
 /* HBM -> registers: 16 B pieces of the 64-key tile whose first row is at
  * `kt` / `vt` (wave-uniform pointers), at this thread's four row offsets. */
-__device__ __forceinline__ void fetch_tile(TileRegs &t, const uint16_t *kt, const uint16_t *vt,
+template <int NP>
+__device__ __forceinline__ void fetch_tile(TileRegs<NP> &t, const uint16_t *kt, const uint16_t *vt,
                                            const uint32_t *off) {
     const char *kc = reinterpret_cast<const char *>(kt), *vc = reinterpret_cast<const char *>(vt);
-    t.k0 = *reinterpret_cast<const u32x4 *>(kc + off[0]);
-    t.v0 = *reinterpret_cast<const u32x4 *>(vc + off[0]);
-    t.k1 = *reinterpret_cast<const u32x4 *>(kc + off[1]);
-    t.v1 = *reinterpret_cast<const u32x4 *>(vc + off[1]);
-    t.k2 = *reinterpret_cast<const u32x4 *>(kc + off[2]);
-    t.v2 = *reinterpret_cast<const u32x4 *>(vc + off[2]);
-    t.k3 = *reinterpret_cast<const u32x4 *>(kc + off[3]);
-    t.v3 = *reinterpret_cast<const u32x4 *>(vc + off[3]);
+#pragma unroll
+    for (int c = 0; c < NP; c++) {
+        t.k[c] = *reinterpret_cast<const u32x4 *>(kc + off[c]);
+        t.v[c] = *reinterpret_cast<const u32x4 *>(vc + off[c]);
+    }
 }
 
 /* Registers -> LDS stage. */
-__device__ __forceinline__ void store_tile(const TileRegs &t, uint16_t *stage, int tid) {
+template <int NP>
+__device__ __forceinline__ void store_tile(const TileRegs<NP> &t, uint16_t *stage, int tid) {
+    constexpr int RSTEP = 64 / NP;
     const int row = tid >> 4, col = (tid & 15) * 8;
     uint16_t *kp = &stage[row * KS + col], *vp = &stage[K_TILE + row * VS + col];
-    *reinterpret_cast<u32x4 *>(kp) = t.k0;
-    *reinterpret_cast<u32x4 *>(vp) = t.v0;
-    *reinterpret_cast<u32x4 *>(kp + 16 * KS) = t.k1;
-    *reinterpret_cast<u32x4 *>(vp + 16 * VS) = t.v1;
-    *reinterpret_cast<u32x4 *>(kp + 32 * KS) = t.k2;
-    *reinterpret_cast<u32x4 *>(vp + 32 * VS) = t.v2;
-    *reinterpret_cast<u32x4 *>(kp + 48 * KS) = t.k3;
-    *reinterpret_cast<u32x4 *>(vp + 48 * VS) = t.v3;
+#pragma unroll
+    for (int c = 0; c < NP; c++) {
+        *reinterpret_cast<u32x4 *>(kp + c * RSTEP * KS) = t.k[c];
+        *reinterpret_cast<u32x4 *>(vp + c * RSTEP * VS) = t.v[c];
+    }
 }
 
 /* Byte offsets of this thread's four rows of a tile starting at key k0; rows
  * past the end are redirected to the last valid row (their scores are masked
  * and their probabilities are exactly zero, so the values never matter). */
-__device__ __forceinline__ void tile_offsets(uint32_t (&off)[4], int tid, int ldi, int k0, int seq_k) {
+template <int NP>
+__device__ __forceinline__ void tile_offsets(uint32_t (&off)[NP], int tid, int ldi, int k0, int seq_k) {
     const int row = tid >> 4, col = (tid & 15) * 8;
+    constexpr int RSTEP = 64 / NP;
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
-        int r = min(row + 16 * c, seq_k - 1 - k0);
+    for (int c = 0; c < NP; c++) {
+        int r = min(row + RSTEP * c, seq_k - 1 - k0);
         off[c] = (uint32_t)(r * ldi + col) * 2u;
     }
 }
 
-template <bool CAUSAL, bool MASK>
-__global__ void __launch_bounds__(THREADS, 2)
+template <int WAVES, bool CAUSAL, bool MASK>
+__global__ void __launch_bounds__(64 * WAVES, 2)
 k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ q,
                const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
                int seq_q, int seq_k, int q_tiles, int total_work, int work_per_xcd,
                int kv_group, float scale_log2, const int *__restrict__ key_mask) {
     extern __shared__ __align__(16) uint16_t lds[];     /* two stages of [K tile | V tile] */
+    constexpr int BM = 32 * WAVES, NP = 16 / WAVES;
 
     /* XCD-aware numbering: hardware deals workgroups round-robin to the 8
      * XCDs, so id%8 is the XCD; give each XCD a contiguous slice of the
@@ -200,23 +205,23 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     /* Row offsets of this thread's 16 B pieces: one set for full tiles, one for
      * the last tile (rows past seq_k redirected to the last valid row). */
     const int last_k0 = (ntiles - 1) * BN;
-    uint32_t off_full[4], off_last[4];
+    uint32_t off_full[NP], off_last[NP];
     tile_offsets(off_full, tid, ldi, 0, BN);
     tile_offsets(off_last, tid, ldi, last_k0, seq_k);
 
     /* ---- prologue: tile 0 -> stage 0, tile 1 -> registers. Tile indices past
      * the end are clamped to the last tile: the copy is redundant but keeps the
      * pipeline free of control flow. ---- */
-    TileRegs tile;
+    TileRegs<NP> tile;
     {
-        uint32_t off[4];
+        uint32_t off[NP];
 #pragma unroll
-        for (int c = 0; c < 4; c++) off[c] = ntiles > 1 ? off_full[c] : off_last[c];
+        for (int c = 0; c < NP; c++) off[c] = ntiles > 1 ? off_full[c] : off_last[c];
         fetch_tile(tile, kbase, vbase, off);
         store_tile(tile, lds, tid);
         const int kn = min(BN, last_k0);
 #pragma unroll
-        for (int c = 0; c < 4; c++) off[c] = kn == last_k0 ? off_last[c] : off_full[c];
+        for (int c = 0; c < NP; c++) off[c] = kn == last_k0 ? off_last[c] : off_full[c];
         fetch_tile(tile, kbase + (size_t)kn * ldi, vbase + (size_t)kn * ldi, off);
     }
     __syncthreads();
@@ -231,9 +236,9 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         {
             const int kn = min(k0 + 2 * BN, last_k0);
             const bool is_last = kn == last_k0;
-            uint32_t off[4];
+            uint32_t off[NP];
 #pragma unroll
-            for (int c = 0; c < 4; c++) off[c] = is_last ? off_last[c] : off_full[c];
+            for (int c = 0; c < NP; c++) off[c] = is_last ? off_last[c] : off_full[c];
             fetch_tile(tile, kbase + (size_t)kn * ldi, vbase + (size_t)kn * ldi, off);
         }
 
@@ -371,21 +376,38 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 }
 
 constexpr size_t LDS_BYTES = 2 * STAGE * sizeof(uint16_t);
+constexpr int CUS = 256;
 
-template <bool C, bool M>
-int launch(hipStream_t st, dim3 grid, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
-           const uint16_t *v, int ldi, int seq_q, int seq_k, int q_tiles, int total, int per_xcd,
-           int kv_group, float scale_log2, const int *key_mask) {
+template <int W, bool C, bool M>
+int launch(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
+           const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads,
+           float scale, const int *key_mask) {
     static bool configured = false;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd128<C, M>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd128<W, C, M>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
         if (e != hipSuccess) return (int)e;
         configured = true;
     }
-    hipLaunchKernelGGL((k_fa_fwd_hd128<C, M>), grid, dim3(THREADS), LDS_BYTES, st, out, ldo, q, k, v, ldi,
-                       seq_q, seq_k, q_tiles, total, per_xcd, kv_group, scale_log2, key_mask);
+    const int q_tiles = (seq_q + 32 * W - 1) / (32 * W);
+    const int total = q_tiles * heads;
+    const int per_xcd = (total + XCDS - 1) / XCDS;
+    hipLaunchKernelGGL((k_fa_fwd_hd128<W, C, M>), dim3(per_xcd * XCDS), dim3(64 * W), LDS_BYTES, st, out, ldo,
+                       q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, heads / kv_heads,
+                       scale * 1.4426950408889634f, key_mask);
     return (int)hipGetLastError();
+}
+
+template <int W>
+int launch_w(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
+             const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads, float scale,
+             int causal, const int *key_mask) {
+    if (causal) {
+        if (key_mask) return launch<W, true, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask);
+        return launch<W, true, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask);
+    }
+    if (key_mask) return launch<W, false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask);
+    return launch<W, false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask);
 }
 
 }  // namespace
@@ -394,17 +416,11 @@ extern "C" int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uin
                                  const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
                                  int seq_k, int heads, int kv_heads, float scale, int causal,
                                  const int *key_mask) {
-    const int q_tiles = (seq_q + BM - 1) / BM;
-    const int total = q_tiles * heads;
-    const int per_xcd = (total + XCDS - 1) / XCDS;
-    const dim3 grid(per_xcd * XCDS);
-    const float scale_log2 = scale * 1.4426950408889634f;
-    const int kv_group = heads / kv_heads;
     hipStream_t st = (hipStream_t)stream;
-    if (causal) {
-        if (key_mask) return launch<true, true>(st, grid, out, ldo, q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, kv_group, scale_log2, key_mask);
-        return launch<true, false>(st, grid, out, ldo, q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, kv_group, scale_log2, key_mask);
-    }
-    if (key_mask) return launch<false, true>(st, grid, out, ldo, q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, kv_group, scale_log2, key_mask);
-    return launch<false, false>(st, grid, out, ldo, q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, kv_group, scale_log2, key_mask);
+    /* 256 queries per workgroup halve the K/V traffic from L2 and the LDS writes per query;
+     * 128 give twice the workgroups when the problem is too small to fill the CUs. */
+    const long wg256 = (long)((seq_q + 255) / 256) * heads;
+    if (wg256 >= CUS)
+        return launch_w<8>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
+    return launch_w<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
 }

@@ -31,6 +31,31 @@ __global__ void __launch_bounds__(256) k_mfma_peak(float *sink, int iters) {
     if (s == 12345.678f) sink[0] = s;
 }
 
+/* The same loop with operands taken from memory (8 x 16 B per lane): the matrix
+ * cores draw more power on real data than on constants, and the clock follows,
+ * so the sustained rate depends on what is multiplied. */
+__global__ void __launch_bounds__(256) k_mfma_data(const uint4 *__restrict__ ops, float *sink, int iters) {
+    f32x16 acc[4];
+    for (int a = 0; a < 4; a++)
+        for (int r = 0; r < 16; r++) acc[a][r] = 0.0f;
+    bf16x8 x[4], y[4];
+    for (int i = 0; i < 4; i++) {
+        x[i] = __builtin_bit_cast(bf16x8, ops[(2 * i) * 256 + threadIdx.x]);
+        y[i] = __builtin_bit_cast(bf16x8, ops[(2 * i + 1) * 256 + threadIdx.x]);
+    }
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x[j], y[(j + a) & 3], acc[a], 0, 0, 0);
+    }
+    float s = 0.0f;
+    for (int a = 0; a < 4; a++)
+        for (int r = 0; r < 16; r++) s += acc[a][r];
+    if (s == 12345.678f) sink[0] = s;
+}
+
 __global__ void __launch_bounds__(256) k_copy(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n) {
     size_t i = (size_t)blockIdx.x * 256 * 4 + threadIdx.x;
 #pragma unroll
@@ -93,6 +118,11 @@ __global__ void __launch_bounds__(256) k_exp(float *sink, int iters) {
 extern "C" {
 int iris_mb_mfma(void *stream, float *sink, int blocks, int iters) {
     hipLaunchKernelGGL(k_mfma_peak, dim3(blocks), dim3(256), 0, (hipStream_t)stream, sink, iters);
+    return (int)hipGetLastError();
+}
+/* ops: device buffer of 8 * 256 * 16 B operand data; iters x 16 MFMAs per wave */
+int iris_mb_mfma_data(void *stream, const void *ops, float *sink, int blocks, int iters) {
+    hipLaunchKernelGGL(k_mfma_data, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const uint4 *)ops, sink, iters);
     return (int)hipGetLastError();
 }
 int iris_mb_copy(void *stream, void *dst, const void *src, size_t bytes) {
