@@ -33,6 +33,13 @@ int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uint16_t *q,
                       const uint16_t *k, const uint16_t *v, int ldi, int seq_q, int seq_k,
                       int heads, int kv_heads, float scale, int causal, const int *key_mask);
 
+/* head_dim 256 or 512 (the VAE's single 512-wide head): the head dim is cut into slices of
+ * 128 that a group of waves shares; same argument conditions as iris_hip_fa_hd128. */
+int iris_hip_fa_sliced(void *stream, uint16_t *out, int ldo, const uint16_t *q,
+                       const uint16_t *k, const uint16_t *v, int ldi, int seq_q, int seq_k,
+                       int heads, int kv_heads, int head_dim, float scale, int causal,
+                       const int *key_mask);
+
 /* Any head_dim <= 512, any stride / alignment / scale. Correctness path. */
 int iris_hip_attention_generic(void *stream, uint16_t *out, int ldo, const uint16_t *q,
                                const uint16_t *k, const uint16_t *v, int ldi, int seq_q,

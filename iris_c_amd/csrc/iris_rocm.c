@@ -182,13 +182,17 @@ void iris_dev_attention(uint16_t *out, int ldo,
         fail(-1, "attention", "need heads % kv_heads == 0, 0 < head_dim <= 512, seq_k >= 0");
         return;
     }
-    int fast = head_dim == 128 && seq_k > 0 && scale > 0.0f && ldi % 8 == 0 && ldo % 4 == 0 &&
-               aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out, 8);
+    int mfma_ok = seq_k > 0 && scale > 0.0f && ldi % 8 == 0 && ldo % 4 == 0 &&
+                  aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out, 8);
     int err;
-    if (fast) {
+    if (mfma_ok && head_dim == 128) {
         g_last_kernel = "fa_hd128";
         err = iris_hip_fa_hd128(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads,
                                 scale, causal != 0, key_mask);
+    } else if (mfma_ok && (head_dim == 256 || head_dim == 512)) {
+        g_last_kernel = "fa_sliced";
+        err = iris_hip_fa_sliced(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads,
+                                 head_dim, scale, causal != 0, key_mask);
     } else {
         g_last_kernel = "attention_generic";
         err = iris_hip_attention_generic(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads,

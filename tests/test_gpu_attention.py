@@ -197,8 +197,57 @@ def test_output_stride_and_interior_pointers(dev, orc, fa):
     assert np.all(out[:, :out_col] == 0x7fc0) and np.all(out[:, out_col + 256:] == 0x7fc0)
 
 
+@pytest.mark.parametrize("hd,heads,kv", [(512, 1, 1), (512, 2, 1), (256, 3, 3), (256, 4, 2)])
+@pytest.mark.parametrize("seq_q,seq_k,causal,masked", [(150, 150, False, False), (1, 1, False, False), (33, 95, False, True),
+                                                         (64, 64, True, False), (257, 257, True, True), (130, 1000, False, False)])
+def test_sliced_kernel_head_dims_256_512(dev, orc, hd, heads, kv, seq_q, seq_k, causal, masked):
+    """head_dim 256 / 512 (the VAE's single 512-wide head) run on the matrix cores too."""
+    buf, ldi = random_case(hd + heads + seq_q, seq_q, seq_k, heads, kv, hd=hd)
+    qd, kd = heads * hd, kv * hd
+    mask = None
+    if masked:
+        mask = (np.random.default_rng(seq_k).random(seq_k) < 0.6).astype(np.int32)
+        mask[0] = 1                                        # every causal row keeps a valid key
+    scale = float(1 / np.sqrt(hd))
+    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
+    assert kernel == "fa_sliced"
+    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
+    assert_close(O.bf16_to_f32(out[:seq_q]), want, f"sliced hd={hd} {seq_q}x{seq_k}")
+
+
+def test_vae_shape_full_size_sampled_rows(dev, orc):
+    """One head of 512 over 4096 tokens (a 512x512 image's mid-block attention, reference
+    iris_vae.c:1112-1124): sampled rows against the oracle, and constant V => constant output."""
+    seq, hd = 4096, 512
+    buf, ldi = random_case(77, seq, seq, 1, 1, hd=hd)
+    scale = float(1 / np.sqrt(hd))
+    out, kernel = dev.attention(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale)
+    assert kernel == "fa_sliced"
+    rows = sample_rows(seq, n=20)
+    want = orc.attention_bf16(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale, rows=rows)
+    assert_close(O.bf16_to_f32(out)[rows], want, "VAE shape sampled")
+    const = buf.copy()
+    const[:, 2 * hd:] = buf[5, 2 * hd:]
+    out2, _ = dev.attention(const, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale)
+    assert_close(O.bf16_to_f32(out2), np.tile(O.bf16_to_f32(buf[5, 2 * hd:]), (seq, 1)), "VAE shape constant V")
+
+
+def test_sliced_kernel_empty_rows_and_large_scores(dev, orc):
+    seq, hd = 100, 512
+    buf, ldi = random_case(21, seq, seq, 1, 1, hd=hd, sigma=3.0)          # |score| up to ~100
+    scale = float(1 / np.sqrt(hd))
+    mask = np.ones(seq, np.int32); mask[:10] = 0
+    out, kernel = dev.attention(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale, True, mask)
+    assert kernel == "fa_sliced"
+    got = O.bf16_to_f32(out)
+    assert np.all(np.isfinite(got)) and np.all(got[:10] == 0.0)
+    want = orc.attention_bf16(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale, True, mask)
+    mx, mean = error_stats(got[10:], want[10:])
+    assert mx <= 0.07 and mean <= 4e-3      # outputs are O(3): same relative bar as 2e-2 on O(1) values
+
+
 @pytest.mark.parametrize("hd,heads,kv,causal,masked", [(64, 4, 4, False, False), (64, 4, 2, True, True),
-                                                       (512, 1, 1, False, False), (96, 2, 1, True, False)])
+                                                       (384, 1, 1, False, False), (96, 2, 1, True, False)])
 def test_generic_kernel_other_head_dims(dev, orc, hd, heads, kv, causal, masked):
     seq = 150
     buf, ldi = random_case(hd + heads, seq, seq, heads, kv, hd=hd)
