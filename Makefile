@@ -18,8 +18,17 @@ CFLAGS   = -O2 -fPIC -Wall -Wextra -std=c11 -I$(CSRC) -Iinclude -I$(ROCM_HOME)/i
 HIP_SRCS = $(CSRC)/qknorm_rope.hip $(CSRC)/fa_fwd_gfx950.hip $(CSRC)/fa_fwd_sliced_gfx950.hip $(CSRC)/attn_generic.hip
 HIP_OBJS = $(HIP_SRCS:.hip=.o)
 
-.PHONY: rocm oracle clean test-cpu test-gpu bench
+.PHONY: rocm oracle clean test-cpu test-gpu bench ctest
 rocm: $(OUT) iris_c_amd/libiris_microbench.so
+
+# C-language parity program: host C over the ABI, checked against the oracle (run by the GPU tests)
+ctest: tests/c_abi_parity.bin
+tests/c_abi_parity.bin: tests/c_abi_parity.c include/iris_dev.h oracle/iris_oracle.h $(OUT) oracle/libiris_oracle.so
+	$(CC) -O2 -Wall -Wextra -std=c11 -Iinclude -Ioracle -o $@ $< -Liris_c_amd -liris_dev -Loracle -liris_oracle \
+	    -Wl,-rpath,'$$ORIGIN/../iris_c_amd' -Wl,-rpath,'$$ORIGIN/../oracle' -Wl,-rpath,$(ROCM_HOME)/lib -lm
+
+oracle/libiris_oracle.so:
+	$(MAKE) -C oracle oracle
 
 # machine-ceiling microbenchmarks used by bench.py only
 iris_c_amd/libiris_microbench.so: $(CSRC)/microbench.hip
@@ -45,4 +54,4 @@ bench:
 	python bench.py
 
 clean:
-	rm -f $(CSRC)/*.o $(OUT) iris_c_amd/libiris_microbench.so
+	rm -f $(CSRC)/*.o $(OUT) iris_c_amd/libiris_microbench.so tests/c_abi_parity.bin
