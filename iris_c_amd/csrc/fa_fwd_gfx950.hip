@@ -1,6 +1,6 @@
 /*
  * Flash-attention forward for gfx950 (MI355X), head_dim 128, bf16 inputs,
- * f32 accumulation on the matrix cores (v_mfma_f32_32x32x16_bf16).
+ * f32 accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16).
  *
  * What it computes (reference iris_dev.h:83-92, iris_cuda.cu:597-682 for the
  * online-softmax recurrence): for every head h and query i
@@ -22,22 +22,34 @@
  *
  * Both products are issued transposed so that a query is a COLUMN of every
  * accumulator: S^T = K Q^T (A = K tile from LDS, B = Q^T held in registers)
- * and O^T += V^T P^T (A = V^T from LDS, B = P^T). In the 32x32 accumulator
- * layout lane l holds column l%32, so each lane carries one query: its
- * running max, its running sum and its rescale factor are plain per-lane
- * scalars, the 32 scores of a 64-key tile that a lane holds all belong to
- * that query, and exp2(S^T) converted to bf16 IS the B operand of the second
- * product -- no LDS round trip, no cross-lane shuffles except one
- * v_permlane32_swap per tile to combine the two half-waves' row maxima.
+ * and O^T += V^T P^T (A = V^T from LDS, B = P^T). In the 16x16 accumulator
+ * layout lane l holds column l%16 and rows 4(l/16) .. +3, so a lane carries
+ * two queries (one per 16-query block), their running max, sum and rescale
+ * factor are per-lane scalars, and exp2(S^T) converted to bf16 IS the B
+ * operand of the second product -- no LDS round trip; the only cross-lane
+ * traffic is one v_permlane16_swap + one v_permlane32_swap per query block
+ * and tile to combine the row maxima of the four lanes that share a query.
  *
- * LDS layout: K tile row-major [64][128+8] bf16 (272 B rows = 16 B x odd, so
- * the 16 consecutive keys a ds_read_b128 phase touches fall in distinct
- * banks). V tile row-major too, [64][128+32] (320 B rows); the V^T operand
- * is produced by the LDS transpose read ds_read_b64_tr_b16, which hands lane
- * i of a 16-lane group column i of a 4-row x 16-column block: four
- * consecutive keys of one head dim, which is exactly the group of keys that
- * four consecutive P^T registers of that lane belong to. With 320 B rows the
- * four rows of a group fall in disjoint banks.
+ * Why 16x16x32 and not 32x32x16: same matrix throughput on paper, but this
+ * GPU is power-limited on real data, and a loop of nothing but MFMAs on
+ * N(0,1) operands sustains about 1.8 PFLOP/s with the 16x16x32 shape
+ * against 1.3 with 32x32x16 (a quarter of the accumulator registers read
+ * and written per flop).
+ *
+ * LDS layout: K and V tiles row-major [64][128+16] bf16, 288 B rows.
+ * ds_read_b128 serves 16 lanes per pass, and a pass is not 16 consecutive
+ * lanes: with lanes 0-3, 12-15, 20-23, 24-27 in one pass (and the other
+ * passes alike) the 16 lanes must fall in distinct 16 B bank windows. The
+ * A operand read has lane l at row l%16, 16 B chunk l/16 (+ constants), so
+ * the window is (row * 288/16 + chunk) % 16 = (2 row + chunk) % 16, which is
+ * a bijection on every such pass; 272 B rows (row + chunk) gave a two-way
+ * conflict on every read. The V^T operand comes from the LDS transpose read
+ * ds_read_b64_tr_b16, which hands lane i of a 16-lane group column i of a
+ * 4-row x 16-column block: four consecutive keys of one head dim, exactly
+ * the keys that four consecutive P^T registers of that lane belong to; it
+ * serves 32 consecutive lanes (8 rows x 32 B) per pass, conflict-free when
+ * the row stride is 32 B mod 256 B. Both hardware counters read zero bank
+ * conflicts with this layout.
  *
  * The running max is only raised when some query of the wave exceeds it by
  * more than 2^8 (the accumulators are then rescaled); otherwise the
@@ -58,15 +70,15 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
 /* A workgroup is WAVES (4 or 8) waves of 32 queries: BM = 32 * WAVES queries, 64 * WAVES threads. */
 constexpr int BN = 64;             /* keys per tile */
 constexpr int HD = 128;
-constexpr int KS = HD + 8;         /* K tile row stride in elements (272 B) */
-constexpr int VS = HD + 32;        /* V tile row stride in elements (320 B) */
+constexpr int KS = HD + 16;         /* K tile row stride in elements (288 B) */
+constexpr int VS = HD + 16;         /* V tile row stride in elements (288 B) */
 constexpr int K_TILE = BN * KS;    /* elements */
 constexpr int V_TILE = BN * VS;
 constexpr int STAGE = K_TILE + V_TILE;
@@ -100,14 +112,20 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
     return d;
 }
 
-/* Max (or sum) of a value with the same lane of the other half-wave. */
-__device__ __forceinline__ float half_swap_max(float v) {
-    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+/* Max (or sum) over the four lanes l%16, l%16+16, +32, +48 (one per 16-lane row); every one
+ * of them gets the result. v_permlane16_swap(x, x) returns rows {0,0,2,2} and {1,1,3,3} of x,
+ * v_permlane32_swap(x, x) rows {0,1,0,1} and {2,3,2,3}. */
+__device__ __forceinline__ float quad_group_max(float v) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    const float t = max3(__uint_as_float(a[0]), __uint_as_float(a[1]), __uint_as_float(a[1]));
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false);
+    return max3(__uint_as_float(b[0]), __uint_as_float(b[1]), __uint_as_float(b[1]));
 }
-__device__ __forceinline__ float half_swap_sum(float v) {
-    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+__device__ __forceinline__ float quad_group_sum(float v) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    const float t = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 /* HBM -> registers: 16 B pieces of the 64-key tile whose first row is at
@@ -170,37 +188,42 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     const int kvh = head / kv_group;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int col = lane & 31, hh = lane >> 5;
-    const int q0 = qt * BM, wq0 = q0 + wave * 32, qrow = wq0 + col;
+    const int li = lane & 15, lg = lane >> 4;       /* 16x16 block: column li, row group lg */
+    const int q0 = qt * BM, wq0 = q0 + wave * 32;
+    const int qrow0 = wq0 + li, qrow1 = qrow0 + 16; /* this lane's two queries (query blocks 0 and 1) */
 
     const uint16_t *kbase = k + (size_t)kvh * HD;
     const uint16_t *vbase = v + (size_t)kvh * HD;
 
-    /* Q^T as B operands: lane (query col, half hh) holds dims 16t + 8hh .. +7. */
-    bf16x8 qb[8];
-    {
-        const uint16_t *qp = q + (size_t)min(qrow, seq_q - 1) * ldi + (size_t)head * HD + 8 * hh;
+    /* Q^T as B operands: for query block nb and k-step ks the lane holds dims 32ks + 8lg .. +7
+     * of query 16nb + li. */
+    bf16x8 qb[2][4];
 #pragma unroll
-        for (int t = 0; t < 8; t++) qb[t] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 16 * t));
+    for (int nb = 0; nb < 2; nb++) {
+        const uint16_t *qp = q + (size_t)min(qrow0 + 16 * nb, seq_q - 1) * ldi + (size_t)head * HD + 8 * lg;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+            qb[nb][ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 32 * ks));
     }
 
-    f32x16 o[4];
+    f32x4 o[8][2];                                   /* O^T: dims 16db + 4lg + r of query block nb */
 #pragma unroll
-    for (int db = 0; db < 4; db++)
+    for (int db = 0; db < 8; db++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f;
+        for (int nb = 0; nb < 2; nb++) o[db][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.0f, 0.0f};
 
     int k_end = seq_k;
     if (CAUSAL) k_end = min(seq_k, q0 + BM);       /* keys beyond the last query of the block are never valid */
     const int ntiles = (k_end + BN - 1) / BN;
 
     /* LDS read addresses (elements, relative to a stage).
-     * K operand: row = key (col [+32]), 16 B at dims 16t + 8hh.
-     * V^T operand: transpose read; lane supplies row 4hh + (lane%16)/4 (+16t, +8)
-     * and columns 16*((lane/16)%2) + 4*(lane%4) (+32db). */
-    const int k_rd = col * KS + 8 * hh;
-    const int v_rd = K_TILE + (4 * hh + ((lane & 15) >> 2)) * VS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+     * K operand (key block mb, k-step ks): row = key 16mb + li, 16 B at dims 32ks + 8lg.
+     * V^T operand (dim block db, k-step ks): transpose read of a 4-key x 16-dim block per
+     * 16-lane group; the lane supplies row 4lg + li/4 (+32ks, +16 for the second half)
+     * and columns 4(li%4) (+16db), and receives the four keys of dim 16db + li. */
+    const int k_rd = li * KS + 8 * lg;
+    const int v_rd = K_TILE + (4 * lg + (li >> 2)) * VS + 4 * (li & 3);
 
     /* Row offsets of this thread's 16 B pieces: one set for full tiles, one for
      * the last tile (rows past seq_k redirected to the last valid row). */
@@ -242,136 +265,147 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             fetch_tile(tile, kbase + (size_t)kn * ldi, vbase + (size_t)kn * ldi, off);
         }
 
-        /* ---- S^T = K Q^T : two 32-key blocks, 8 k-steps over the head dim.
+        /* ---- S^T = K Q^T : 4 key blocks x 2 query blocks of 16x16, 4 k-steps of 32 dims.
          * All 16 A operands are requested from LDS up front so their latency
-         * overlaps instead of gating every MFMA. ---- */
-        f32x16 s0, s1;
+         * overlaps instead of gating every MFMA; each feeds two MFMAs. ---- */
+        f32x4 s[4][2];
         {
-            u32x4 ka[8], kb[8];
+            u32x4 ka[4][4];
 #pragma unroll
-            for (int t = 0; t < 8; t++) {
-                ka[t] = *reinterpret_cast<const u32x4 *>(&cur[k_rd + 16 * t]);
-                kb[t] = *reinterpret_cast<const u32x4 *>(&cur[k_rd + 32 * KS + 16 * t]);
-            }
+            for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++)
+                    ka[mb][ks] = *reinterpret_cast<const u32x4 *>(&cur[k_rd + 16 * mb * KS + 32 * ks]);
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(1);
-            const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[0]), qb[0], zero, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kb[0]), qb[0], zero, 0, 0, 0);
+            const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int t = 1; t < 8; t++) {
-                s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[t]), qb[t], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kb[t]), qb[t], s1, 0, 0, 0);
-            }
+            for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                for (int nb = 0; nb < 2; nb++)
+                    s[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[mb][0]), qb[nb][0], zero, 0, 0, 0);
+#pragma unroll
+            for (int ks = 1; ks < 4; ks++)
+#pragma unroll
+                for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                    for (int nb = 0; nb < 2; nb++)
+                        s[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[mb][ks]), qb[nb][ks], s[mb][nb], 0, 0, 0);
             __builtin_amdgcn_s_setprio(0);
         }
-        /* register r of block b holds key k0 + 32b + 8(r/4) + 4hh + r%4 for query qrow */
+        /* s[mb][nb][r] is key k0 + 16mb + 4lg + r against query 16nb + li of the wave */
 
         /* ---- validity: range / key mask (wave-uniform 64-bit set), causal (per lane) ---- */
         unsigned long long valid = ~0ull;
         if (k0 + BN > seq_k) valid = (1ull << (seq_k - k0)) - 1ull;
         if (MASK) valid &= __ballot((k0 + lane < seq_k) && key_mask[min(k0 + lane, seq_k - 1)] != 0);
         if (valid != ~0ull) {
-            const unsigned long long mine = valid >> (4 * hh);
-            const uint32_t lo = (uint32_t)mine, hi = (uint32_t)(mine >> 32);
+            const unsigned long long mine = valid >> (4 * lg);
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int bit = 8 * (r >> 2) + (r & 3);
-                if (!((lo >> bit) & 1u)) s0[r] = -INFINITY;
-                if (!((hi >> bit) & 1u)) s1[r] = -INFINITY;
-            }
+            for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (!((mine >> (16 * mb + r)) & 1ull)) { s[mb][0][r] = -INFINITY; s[mb][1][r] = -INFINITY; }
         }
         if (CAUSAL && k0 + BN - 1 > wq0) {
-            const int lim = qrow - k0 - 4 * hh;    /* key offset const_r valid iff const_r <= lim */
+            const int lim0 = qrow0 - k0 - 4 * lg;      /* key offset 16mb + r valid iff <= lim */
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int koff = 8 * (r >> 2) + (r & 3);
-                if (koff > lim) s0[r] = -INFINITY;
-                if (koff + 32 > lim) s1[r] = -INFINITY;
+            for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    if (16 * mb + r > lim0) s[mb][0][r] = -INFINITY;
+                    if (16 * mb + r > lim0 + 16) s[mb][1][r] = -INFINITY;
+                }
+        }
+
+        /* ---- online softmax: the lane holds 16 of the 64 scores of each of its two queries;
+         * the other three quarters sit in the lanes 16, 32 and 48 away ---- */
+        float mx[2];
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
+            const float t1 = max3(s[0][nb][0], s[0][nb][1], s[0][nb][2]);
+            const float t2 = max3(s[0][nb][3], s[1][nb][0], s[1][nb][1]);
+            const float t3 = max3(s[1][nb][2], s[1][nb][3], s[2][nb][0]);
+            const float t4 = max3(s[2][nb][1], s[2][nb][2], s[2][nb][3]);
+            const float t5 = max3(s[3][nb][0], s[3][nb][1], s[3][nb][2]);
+            const float u1 = max3(t1, t2, t3), u2 = max3(t4, t5, s[3][nb][3]);
+            mx[nb] = quad_group_max(max3(u1, u2, u2)) * scale_log2;
+        }
+
+        if (__any(mx[0] > m_run[0] + RESCALE_THRESHOLD || mx[1] > m_run[1] + RESCALE_THRESHOLD)) {
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++) {
+                const float m_new = fmaxf(m_run[nb], mx[nb]);
+                const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - (m_new == -INFINITY ? 0.0f : m_new));
+                m_run[nb] = m_new;
+                l_run[nb] *= alpha;
+#pragma unroll
+                for (int db = 0; db < 8; db++) o[db][nb] *= alpha;
             }
         }
 
-        /* ---- online softmax, one query per lane ---- */
-        float mx = max3(s0[0], s0[1], s1[0]);
-        mx = max3(mx, s1[1], s0[2]);
+        /* P^T as B operands: k-step ks covers keys 32ks .. 32ks+31, of which this lane's 8 are
+         * 32ks + 4lg + r (key block 2ks) and 32ks + 16 + 4lg + r (key block 2ks+1). */
+        u32x4 pw[2][2];
 #pragma unroll
-        for (int r = 3; r < 16; r += 2) mx = max3(mx, s0[r], s0[r + 1 < 16 ? r + 1 : r]);
+        for (int nb = 0; nb < 2; nb++) {
+            const float neg_m = m_run[nb] == -INFINITY ? 0.0f : -m_run[nb];   /* finite while every key so far is masked */
+            float psum = 0.0f;
 #pragma unroll
-        for (int r = 2; r < 16; r += 2) mx = max3(mx, s1[r], s1[r + 1]);
-        mx = half_swap_max(mx) * scale_log2;
-
-        if (__any(mx > m_run + RESCALE_THRESHOLD)) {
-            const float m_new = fmaxf(m_run, mx);
-            const float alpha = __builtin_amdgcn_exp2f(m_run - (m_new == -INFINITY ? 0.0f : m_new));
-            m_run = m_new;
-            l_run *= alpha;
+            for (int ks = 0; ks < 2; ks++) {
+                float p[8];
 #pragma unroll
-            for (int db = 0; db < 4; db++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) o[db][r] *= alpha;
-        }
-        const float neg_m = m_run == -INFINITY ? 0.0f : -m_run;   /* finite while every key so far is masked */
-
-        float psum0 = 0.0f, psum1 = 0.0f;
-        uint32_t pw[16];                            /* P^T as bf16 pairs: pw[4*t + j] = k-step t, elements 2j, 2j+1 */
-#pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-            float p0 = __builtin_amdgcn_exp2f(fmaf(s0[r], scale_log2, neg_m));
-            float p1 = __builtin_amdgcn_exp2f(fmaf(s0[r + 1], scale_log2, neg_m));
-            float p2 = __builtin_amdgcn_exp2f(fmaf(s1[r], scale_log2, neg_m));
-            float p3 = __builtin_amdgcn_exp2f(fmaf(s1[r + 1], scale_log2, neg_m));
-            psum0 += p0 + p1;
-            psum1 += p2 + p3;
-            pw[r >> 1] = pack_bf16(p0, p1);
-            pw[8 + (r >> 1)] = pack_bf16(p2, p3);
-        }
-        l_run += psum0 + psum1;                     /* per half-wave partial; halves are added at the end */
-
-        /* ---- O^T += V^T P^T : 4 k-steps of 16 keys x 4 dim blocks; the V^T
-         * operands of two k-steps are requested together ---- */
-#pragma unroll
-        for (int tp = 0; tp < 4; tp += 2) {
-            s16x4 lo[2][4], hi[2][4];
-#pragma unroll
-            for (int u = 0; u < 2; u++)
-#pragma unroll
-                for (int db = 0; db < 4; db++) {
-                    const uint16_t *vp = &cur[v_rd + 16 * (tp + u) * VS + 32 * db];
-                    lo[u][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp));
-                    hi[u][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 8 * VS));
+                for (int r = 0; r < 4; r++) {
+                    p[r] = __builtin_amdgcn_exp2f(fmaf(s[2 * ks][nb][r], scale_log2, neg_m));
+                    p[4 + r] = __builtin_amdgcn_exp2f(fmaf(s[2 * ks + 1][nb][r], scale_log2, neg_m));
                 }
+                pw[ks][nb] = u32x4{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
+                psum += ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+            }
+            l_run[nb] += psum;                      /* per lane-group partial; the four are added at the end */
+        }
+
+        /* ---- O^T += V^T P^T : 2 k-steps of 32 keys x 8 dim blocks x 2 query blocks; the V^T
+         * operands of a k-step are requested together ---- */
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            s16x4 lo[8], hi[8];
+#pragma unroll
+            for (int db = 0; db < 8; db++) {
+                const uint16_t *vp = &cur[v_rd + 32 * ks * VS + 16 * db];
+                lo[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp));
+                hi[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 16 * VS));
+            }
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(1);
+            const bf16x8 pb0 = __builtin_bit_cast(bf16x8, pw[ks][0]), pb1 = __builtin_bit_cast(bf16x8, pw[ks][1]);
 #pragma unroll
-            for (int u = 0; u < 2; u++) {
-                const int t = tp + u;
-                uint4 praw = make_uint4(pw[4 * t], pw[4 * t + 1], pw[4 * t + 2], pw[4 * t + 3]);
-                bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
-#pragma unroll
-                for (int db = 0; db < 4; db++) {
-                    s16x8 both = __builtin_shufflevector(lo[u][db], hi[u][db], 0, 1, 2, 3, 4, 5, 6, 7);
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pb, o[db], 0, 0, 0);
-                }
+            for (int db = 0; db < 8; db++) {
+                s16x8 both = __builtin_shufflevector(lo[db], hi[db], 0, 1, 2, 3, 4, 5, 6, 7);
+                o[db][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb0, o[db][0], 0, 0, 0);
+                o[db][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb1, o[db][1], 0, 0, 0);
             }
             __builtin_amdgcn_s_setprio(0);
         }
         lds_barrier();
     }
 
-    /* ---- normalise and store: lane holds dims 32db + 8g + 4hh + {0..3} of query qrow ---- */
-    const float l_tot = half_swap_sum(l_run);
-    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-    if (qrow < seq_q) {
-        uint16_t *op = out + (size_t)qrow * ldo + (size_t)head * HD + 4 * hh;
+    /* ---- normalise and store: the lane holds dims 16db + 4lg + {0..3} of its two queries ---- */
 #pragma unroll
-        for (int db = 0; db < 4; db++)
+    for (int nb = 0; nb < 2; nb++) {
+        const float l_tot = quad_group_sum(l_run[nb]);
+        const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+        const int qrow = qrow0 + 16 * nb;
+        if (qrow < seq_q) {
+            uint16_t *op = out + (size_t)qrow * ldo + (size_t)head * HD + 4 * lg;
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
+            for (int db = 0; db < 8; db++) {
                 uint2 w;
-                w.x = pack_bf16(o[db][4 * g] * inv, o[db][4 * g + 1] * inv);
-                w.y = pack_bf16(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
-                *reinterpret_cast<uint2 *>(op + 32 * db + 8 * g) = w;
+                w.x = pack_bf16(o[db][nb][0] * inv, o[db][nb][1] * inv);
+                w.y = pack_bf16(o[db][nb][2] * inv, o[db][nb][3] * inv);
+                *reinterpret_cast<uint2 *>(op + 16 * db) = w;
             }
+        }
     }
 }
 
