@@ -203,6 +203,7 @@ def microbench_lib():
     mb = C.CDLL(os.path.join(ROOT, "iris_c_amd", "libiris_microbench.so"))
     mb.iris_mb_mfma.argtypes = [_vp, _vp, C.c_int, C.c_int]
     mb.iris_mb_mfma_data.argtypes = [_vp, _vp, _vp, C.c_int, C.c_int]
+    mb.iris_mb_mfma_data16.argtypes = [_vp, _vp, _vp, C.c_int, C.c_int]
     mb.iris_mb_copy.argtypes = [_vp, _vp, _vp, C.c_size_t]
     mb.iris_mb_rmw.argtypes = [_vp, _vp, C.c_size_t]
     return mb
@@ -236,6 +237,9 @@ def machine_ceilings(dev, hip, stream):
     mb.iris_mb_mfma_data(stream, ops, sink, blocks, 16)
     ms2 = min(event_time(hip, stream, lambda i: mb.iris_mb_mfma_data(stream, ops, sink, blocks, it2), 1) for _ in range(3))
     mfma_data = blocks * 4 * it2 * 16 * 32768 / ms2 / 1e9
+    mb.iris_mb_mfma_data16(stream, ops, sink, blocks, 16)
+    ms3 = min(event_time(hip, stream, lambda i: mb.iris_mb_mfma_data16(stream, ops, sink, blocks, it2), 1) for _ in range(3))
+    mfma_data16 = blocks * 4 * it2 * 32 * 16384 / ms3 / 1e9
     n = 1 << 30
     a, b = lib.iris_dev_alloc(n), lib.iris_dev_alloc(n)
     assert a and b
@@ -248,9 +252,12 @@ def machine_ceilings(dev, hip, stream):
     return {"mfma_only_tflops": round(mfma, 1), "mfma_only_frac_of_peak": round(mfma / PEAK_BF16_TFLOPS, 4),
             "mfma_only_normal_data_tflops": round(mfma_data, 1),
             "mfma_only_normal_data_frac_of_peak": round(mfma_data / PEAK_BF16_TFLOPS, 4),
+            "mfma16x16x32_only_normal_data_tflops": round(mfma_data16, 1),
+            "mfma16x16x32_only_normal_data_frac_of_peak": round(mfma_data16 / PEAK_BF16_TFLOPS, 4),
             "copy_1gib_gbps": round(2 * n / cp / 1e6, 1), "inplace_update_1gib_gbps": round(2 * n / rw / 1e6, 1),
-            "note": "measured ceilings of this GPU: a pure MFMA loop on constant operands (short burst) and on "
-                    "N(0,1) operands (sustained; the clock drops with the data-dependent power draw), and "
+            "note": "measured ceilings of this GPU: a pure 32x32x16 MFMA loop on constant operands (short burst), "
+                    "the same and the 16x16x32 shape (the one the attention kernel uses) on N(0,1) operands "
+                    "(sustained; the clock drops with the data-dependent power draw), and "
                     "streaming 16 B per lane, bytes counted read + written"}
 
 

@@ -278,6 +278,85 @@ class Oracle:
         return out
 
 
+    # ---- the other device operators (iris_oracle_ops.c) ----
+    def dev_linear(self, x, W):
+        """x bf16 [rows, in], W bf16 [out, in] -> f32 [rows, out]."""
+        rows, k = x.shape
+        out = np.empty((rows, W.shape[0]), np.float32)
+        self.lib.orc_dev_linear(_ptr(out), _ptr(x), _ptr(W), _i(rows), _i(k), _i(W.shape[0]))
+        return out
+
+    def dev_layer_norm_mod(self, x, shift, scale, eps):
+        out = np.empty(x.shape, np.uint16)
+        self.lib.orc_dev_layer_norm_mod(_ptr(out), _ptr(x), _ptr(shift), _ptr(scale), _i(x.shape[0]), _i(x.shape[1]), _f(eps))
+        return out
+
+    def dev_rms_norm_mod(self, x, w, scale, eps):
+        out = np.empty(x.shape, np.uint16)
+        self.lib.orc_dev_rms_norm_mod(_ptr(out), _ptr(x), _ptr(w), _ptr(scale), _i(x.shape[0]), _i(x.shape[1]), _f(eps))
+        return out
+
+    def dev_rms_norm_residual(self, x, a, w, gate, eps):
+        x = x.copy()
+        self.lib.orc_dev_rms_norm_residual(_ptr(x), _ptr(a), _ptr(w), _ptr(gate), _i(x.shape[0]), _i(x.shape[1]), _f(eps))
+        return x
+
+    def dev_swiglu(self, gate_up, cols, ldo=None):
+        """gate_up bf16 [rows, ldi] with gate at column 0 and up at column `cols`."""
+        rows, ldi = gate_up.shape
+        ldo = ldo or cols
+        out = np.zeros((rows, ldo), np.uint16)
+        flat = gate_up.reshape(-1)
+        self.lib.orc_dev_swiglu(_ptr(out), _i(ldo), _ptr(flat), C.c_void_p(flat.ctypes.data + 2 * cols), _i(ldi), _i(rows), _i(cols))
+        return out
+
+    def dev_residual(self, x, a, gate):
+        x = x.copy()
+        self.lib.orc_dev_residual(_ptr(x), _ptr(a), _ptr(gate), _i(x.shape[0]), _i(x.shape[1]))
+        return x
+
+    def dev_silu(self, x):
+        x = np.ascontiguousarray(x, np.float32).copy()
+        self.lib.orc_dev_silu(_ptr(x), C.c_size_t(x.size))
+        return x
+
+    def dev_add(self, x, a):
+        x = x.copy()
+        self.lib.orc_dev_add(_ptr(x), _ptr(a), C.c_size_t(x.size))
+        return x
+
+    def dev_add_bias(self, y, bias):
+        y = y.copy()
+        self.lib.orc_dev_add_bias(_ptr(y), _ptr(bias), _i(y.shape[0]), _i(y.shape[1]))
+        return y
+
+    def dev_fill_rows(self, row, rows):
+        out = np.empty((rows, row.size), np.float32)
+        self.lib.orc_dev_fill_rows(_ptr(out), _ptr(row), _i(rows), _i(row.size))
+        return out
+
+    def dev_conv2d(self, img, w, bias, h, width, k, stride, pad_before, pad_after):
+        """img f32 [h*width, cin], w bf16 [cout, k*k*cin] -> f32 [oh*ow, cout]."""
+        cin, cout = img.shape[1], w.shape[0]
+        oh = (h + pad_before + pad_after - k) // stride + 1
+        ow = (width + pad_before + pad_after - k) // stride + 1
+        out = np.empty((oh * ow, cout), np.float32)
+        self.lib.orc_dev_conv2d(_ptr(out), _ptr(img), _ptr(w), _ptr(bias), _i(h), _i(width), _i(cin), _i(cout), _i(k),
+                                _i(stride), _i(pad_before), _i(pad_after))
+        return out
+
+    def dev_group_norm(self, img, gamma, beta, groups, eps, silu):
+        out = np.empty(img.shape, np.float32)
+        self.lib.orc_dev_group_norm(_ptr(out), _ptr(img), _ptr(gamma), _ptr(beta), _i(img.shape[0]), _i(img.shape[1]),
+                                    _i(groups), _f(eps), _i(int(silu)))
+        return out
+
+    def dev_upsample2x(self, img, h, width):
+        out = np.empty((4 * h * width, img.shape[1]), np.float32)
+        self.lib.orc_dev_upsample2x(_ptr(out), _ptr(img), _i(h), _i(width), _i(img.shape[1]))
+        return out
+
+
 class CpuBaseline:
     """libiris_cpu_baseline.so: the reference's BLAS-build CPU structure, for timing."""
 

@@ -35,6 +35,8 @@
  *                               causal, GQA), compiled zi_attention core
  *   orc_head_norm_rope_bf16     composition of the pinned pieces; device
  *                               semantics iris_cuda.cu:402-420
+ *   orc_dev_*                   the other device operators: see the list
+ *                               at the top of iris_oracle_ops.c
  */
 #ifndef IRIS_ORACLE_H
 #define IRIS_ORACLE_H
@@ -151,6 +153,27 @@ void orc_attention_bf16_rows(float *out, const uint16_t *q, const uint16_t *k,
                              const uint16_t *v, int ldi, const int *rows, int nrows, int seq_k,
                              int heads, int kv_heads, int head_dim, float scale, int causal,
                              const int *key_mask);
+
+/* ---- the remaining device operators (iris_oracle_ops.c; reference iris_dev.h:45-127) ---- */
+void orc_dev_linear(float *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out);
+void orc_dev_layer_norm_mod(uint16_t *out, const float *x, const float *shift, const float *scale,
+                            int rows, int dim, float eps);
+void orc_dev_rms_norm_mod(uint16_t *out, const float *x, const float *w, const float *scale,
+                          int rows, int dim, float eps);
+void orc_dev_rms_norm_residual(float *x, const float *a, const float *w, const float *gate,
+                               int rows, int dim, float eps);
+void orc_dev_swiglu(uint16_t *out, int ldo, const uint16_t *gate, const uint16_t *up, int ldi,
+                    int rows, int cols);
+void orc_dev_residual(float *x, const float *a, const float *gate, int rows, int dim);
+void orc_dev_silu(float *x, size_t n);
+void orc_dev_add(float *x, const float *a, size_t n);
+void orc_dev_add_bias(float *y, const float *bias, int rows, int cols);
+void orc_dev_fill_rows(float *out, const float *row, int rows, int dim);
+void orc_dev_conv2d(float *out, const float *in, const uint16_t *w, const float *bias, int h, int width,
+                    int cin, int cout, int k, int stride, int pad_before, int pad_after);
+void orc_dev_group_norm(float *out, const float *in, const float *gamma, const float *beta, int hw, int c,
+                        int groups, float eps, int silu);
+void orc_dev_upsample2x(float *out, const float *in, int h, int width, int c);
 
 #ifdef __cplusplus
 }
