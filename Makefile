@@ -15,7 +15,8 @@ HIPFLAGS = -O3 --offload-arch=$(GPU_ARCH) -fPIC -std=c++17 -Xclang -target-featu
            -I$(CSRC) -Iinclude
 CFLAGS   = -O2 -fPIC -Wall -Wextra -std=c11 -I$(CSRC) -Iinclude -I$(ROCM_HOME)/include
 
-HIP_SRCS = $(CSRC)/qknorm_rope.hip $(CSRC)/fa_fwd_gfx950.hip $(CSRC)/fa_fwd_sliced_gfx950.hip $(CSRC)/attn_generic.hip
+HIP_SRCS = $(CSRC)/qknorm_rope.hip $(CSRC)/fa_fwd_gfx950.hip $(CSRC)/fa_fwd_sliced_gfx950.hip $(CSRC)/attn_generic.hip \
+           $(CSRC)/ew_norm_ops.hip $(CSRC)/gemm_conv_gfx950.hip
 HIP_OBJS = $(HIP_SRCS:.hip=.o)
 
 .PHONY: rocm oracle clean test-cpu test-gpu bench ctest

@@ -1,5 +1,6 @@
 /*
- * Device (GPU) compute API of the attention hot path, MI355X (gfx950) backend.
+ * Device (GPU) compute API, MI355X (gfx950) backend: the attention hot path and
+ * the other operators of the reference's device header.
  *
  * This is the C ABI of libiris_dev.so. Every declaration below that cites
  * the reference header keeps that header's name, argument order, units and
@@ -67,6 +68,58 @@ void iris_dev_attention(uint16_t *out, int ldo,
                         int ldi, int seq_q, int seq_k, int heads, int kv_heads,
                         int head_dim, float scale, int causal,
                         const int *key_mask);
+
+/* ---- the other operators of the device API (reference iris_dev.h:45-72, 94-127) ----
+ * Same names, arguments and meaning as the reference; each one enqueues on the
+ * library's stream. */
+
+/* dst[i] = bf16(src[i]) (reference iris_dev.h:45-46) */
+void iris_dev_f32_to_bf16(uint16_t *dst, const float *src, size_t n);
+
+/* y[rows, out] = x[rows, in] @ W[out, in]^T: bf16 inputs, f32 accumulation, f32 or bf16
+ * output; all matrices contiguous (reference iris_dev.h:48-53) */
+void iris_dev_linear_f32(float *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out);
+void iris_dev_linear_bf16(uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out);
+
+/* out = LayerNorm(x) * (1 + scale) + shift, no affine parameters; shift / scale [dim],
+ * either may be NULL (reference iris_dev.h:55-59) */
+void iris_dev_layer_norm_mod(uint16_t *out, const float *x, const float *shift, const float *scale,
+                             int rows, int dim, float eps);
+/* out = RMSNorm(x) * w (reference iris_dev.h:61-63) */
+void iris_dev_rms_norm(uint16_t *out, const float *x, const float *w, int rows, int dim, float eps);
+/* out = RMSNorm(x) * w * (1 + scale), scale optional (reference iris_dev.h:65-68) */
+void iris_dev_rms_norm_mod(uint16_t *out, const float *x, const float *w, const float *scale,
+                           int rows, int dim, float eps);
+/* x += tanh(gate) * RMSNorm(a) * w in f32; gate [dim] may be NULL (reference iris_dev.h:70-73) */
+void iris_dev_rms_norm_residual(float *x, const float *a, const float *w, const float *gate,
+                                int rows, int dim, float eps);
+
+/* out[r, c] = silu(gate[r, c]) * up[r, c]; gate / up row stride ldi, out row stride ldo
+ * (reference iris_dev.h:94-97) */
+void iris_dev_swiglu(uint16_t *out, int ldo, const uint16_t *gate, const uint16_t *up, int ldi,
+                     int rows, int cols);
+/* x[r, c] += gate[c] * a[r, c], or x += a when gate is NULL (reference iris_dev.h:99-101) */
+void iris_dev_residual(float *x, const float *a, const float *gate, int rows, int dim);
+
+/* elementwise helpers on f32 vectors (reference iris_dev.h:103-107) */
+void iris_dev_silu(float *x, size_t n);
+void iris_dev_add(float *x, const float *a, size_t n);                    /* x += a */
+void iris_dev_add_bias(float *y, const float *bias, int rows, int cols);  /* y[r, c] += bias[c] */
+void iris_dev_fill_rows(float *out, const float *row, int rows, int dim); /* out[r, c] = row[c] */
+
+/* k x k convolution of a channels-last f32 image [h * width, cin] into [oh * ow, cout] with
+ * zero padding of pad_before / pad_after pixels on each axis,
+ *   oh = (h + pad_before + pad_after - k) / stride + 1 (same for ow),
+ * w: bf16 [cout, k * k * cin] in (ky, kx, c) order, bias may be NULL (reference iris_dev.h:111-121) */
+void iris_dev_conv2d(float *out, const float *in, const uint16_t *w, const float *bias,
+                     int h, int width, int cin, int cout, int k, int stride,
+                     int pad_before, int pad_after);
+/* GroupNorm over [hw, c] with affine gamma / beta [c], optionally followed by SiLU
+ * (reference iris_dev.h:123-126) */
+void iris_dev_group_norm(float *out, const float *in, const float *gamma, const float *beta,
+                         int hw, int c, int groups, float eps, int silu);
+/* nearest-neighbour 2x upsampling of [h * w, c] into [2h * 2w, c] (reference iris_dev.h:128-129) */
+void iris_dev_upsample2x(float *out, const float *in, int h, int width, int c);
 
 /* ---- additions (no counterpart in the reference header) ---- */
 

@@ -28,6 +28,22 @@ ABI = {
     "iris_dev_sync": (None, []),
     "iris_dev_head_norm_rope": (None, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _i]),
     "iris_dev_attention": (None, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp]),
+    "iris_dev_f32_to_bf16": (None, [_vp, _vp, _sz]),
+    "iris_dev_linear_f32": (None, [_vp, _vp, _vp, _i, _i, _i]),
+    "iris_dev_linear_bf16": (None, [_vp, _vp, _vp, _i, _i, _i]),
+    "iris_dev_layer_norm_mod": (None, [_vp, _vp, _vp, _vp, _i, _i, _f]),
+    "iris_dev_rms_norm": (None, [_vp, _vp, _vp, _i, _i, _f]),
+    "iris_dev_rms_norm_mod": (None, [_vp, _vp, _vp, _vp, _i, _i, _f]),
+    "iris_dev_rms_norm_residual": (None, [_vp, _vp, _vp, _vp, _i, _i, _f]),
+    "iris_dev_swiglu": (None, [_vp, _i, _vp, _vp, _i, _i, _i]),
+    "iris_dev_residual": (None, [_vp, _vp, _vp, _i, _i]),
+    "iris_dev_silu": (None, [_vp, _sz]),
+    "iris_dev_add": (None, [_vp, _vp, _sz]),
+    "iris_dev_add_bias": (None, [_vp, _vp, _i, _i]),
+    "iris_dev_fill_rows": (None, [_vp, _vp, _i, _i]),
+    "iris_dev_conv2d": (None, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i]),
+    "iris_dev_group_norm": (None, [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _i]),
+    "iris_dev_upsample2x": (None, [_vp, _vp, _i, _i, _i]),
     "iris_dev_head_norm_rope_qk": (None, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i]),
     "iris_dev_stream": (_vp, []),
     "iris_dev_last_error": (_i, []),

@@ -1,0 +1,376 @@
+/*
+ * Elementwise and normalisation operators of the device API for gfx950
+ * (reference iris_dev.h:45-107, 123-129; kernels iris_cuda.cu:271-400, 943-946,
+ * 1018-1087). All of them are HBM-bound: one pass over the data with 16-byte
+ * accesses per lane where the pointers and sizes allow it, a scalar form of
+ * the same kernel otherwise.
+ *
+ * Row normalisations use one workgroup (256 threads) per row and keep the
+ * row in registers between the statistics and the write (rows up to 4096
+ * floats; longer rows are read again, from cache). Statistics follow the
+ * reference: LayerNorm takes the mean first and the variance about it.
+ */
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "iris_kernels_hip.h"
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+namespace {
+
+constexpr int EW_THREADS = 256;
+constexpr int ROW_THREADS = 256;
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    f32x2 p = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2));
+}
+__device__ __forceinline__ uint16_t to_bf16(float v) { return (uint16_t)(pack_bf16(v, 0.0f) & 0xffffu); }
+__device__ __forceinline__ float bf_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+__device__ __forceinline__ float silu(float v) { return v / (1.0f + __expf(-v)); }
+
+inline unsigned blocks_for(size_t n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
+
+/* ---------------------------------------------------------------- elementwise */
+
+enum EwOp { OP_SILU, OP_ADD, OP_ADD_ROW, OP_MULADD_ROW, OP_FILL_ROW };
+
+/* x[i] = f(x[i], a[i] or row[i % dim]); VEC = floats per thread (4: all pointers 16-byte
+ * aligned and n, dim multiples of 4; 1 otherwise). */
+template <int OP, int VEC>
+__global__ void __launch_bounds__(EW_THREADS)
+k_ew(float *__restrict__ x, const float *__restrict__ a, const float *__restrict__ row, int dim, size_t n) {
+    const size_t i = ((size_t)blockIdx.x * EW_THREADS + threadIdx.x) * VEC;
+    if (i >= n) return;
+    float xv[VEC], av[VEC], rv[VEC];
+    if (VEC == 4) {
+        if (OP != OP_FILL_ROW) *reinterpret_cast<float4 *>(xv) = *reinterpret_cast<const float4 *>(x + i);
+        if (OP == OP_ADD || OP == OP_MULADD_ROW) *reinterpret_cast<float4 *>(av) = *reinterpret_cast<const float4 *>(a + i);
+        if (OP == OP_ADD_ROW || OP == OP_MULADD_ROW || OP == OP_FILL_ROW)
+            *reinterpret_cast<float4 *>(rv) = *reinterpret_cast<const float4 *>(row + i % dim);
+    } else {
+        if (OP != OP_FILL_ROW) xv[0] = x[i];
+        if (OP == OP_ADD || OP == OP_MULADD_ROW) av[0] = a[i];
+        if (OP == OP_ADD_ROW || OP == OP_MULADD_ROW || OP == OP_FILL_ROW) rv[0] = row[i % dim];
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+        if (OP == OP_SILU) xv[j] = silu(xv[j]);
+        if (OP == OP_ADD) xv[j] += av[j];
+        if (OP == OP_ADD_ROW) xv[j] += rv[j];
+        if (OP == OP_MULADD_ROW) xv[j] = fmaf(rv[j], av[j], xv[j]);
+        if (OP == OP_FILL_ROW) xv[j] = rv[j];
+    }
+    if (VEC == 4) *reinterpret_cast<float4 *>(x + i) = *reinterpret_cast<float4 *>(xv);
+    else x[i] = xv[0];
+}
+
+inline bool al16(const void *p) { return p == nullptr || ((uintptr_t)p & 15) == 0; }
+
+template <int OP>
+int launch_ew(hipStream_t st, float *x, const float *a, const float *row, int dim, size_t n) {
+    if (!n) return 0;
+    const bool vec = al16(x) && al16(a) && al16(row) && n % 4 == 0 && (dim <= 0 || dim % 4 == 0);
+    if (vec) hipLaunchKernelGGL((k_ew<OP, 4>), dim3(blocks_for(n, EW_THREADS * 4)), dim3(EW_THREADS), 0, st, x, a, row, dim > 0 ? dim : 4, n);
+    else hipLaunchKernelGGL((k_ew<OP, 1>), dim3(blocks_for(n, EW_THREADS)), dim3(EW_THREADS), 0, st, x, a, row, dim > 0 ? dim : 1, n);
+    return (int)hipGetLastError();
+}
+
+template <int VEC>
+__global__ void __launch_bounds__(EW_THREADS)
+k_f32_to_bf16(uint16_t *__restrict__ dst, const float *__restrict__ src, size_t n) {
+    const size_t i = ((size_t)blockIdx.x * EW_THREADS + threadIdx.x) * VEC;
+    if (i >= n) return;
+    if (VEC == 8) {
+        const float4 a = *reinterpret_cast<const float4 *>(src + i), b = *reinterpret_cast<const float4 *>(src + i + 4);
+        *reinterpret_cast<uint4 *>(dst + i) = make_uint4(pack_bf16(a.x, a.y), pack_bf16(a.z, a.w), pack_bf16(b.x, b.y), pack_bf16(b.z, b.w));
+    } else {
+        dst[i] = to_bf16(src[i]);
+    }
+}
+
+/* out[r, c] = silu(gate[r, c]) * up[r, c] on bf16 rows with strides */
+template <int VEC>
+__global__ void __launch_bounds__(EW_THREADS)
+k_swiglu(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ gate, const uint16_t *__restrict__ up,
+         int ldi, int cols, size_t n) {
+    const size_t i = ((size_t)blockIdx.x * EW_THREADS + threadIdx.x) * VEC;
+    if (i >= n) return;
+    const size_t r = i / cols, c = i % cols;
+    if (VEC == 8) {
+        const uint4 g = *reinterpret_cast<const uint4 *>(gate + r * ldi + c), u = *reinterpret_cast<const uint4 *>(up + r * ldi + c);
+        const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) o[j] = pack_bf16(silu(bf_lo(gw[j])) * bf_lo(uw[j]), silu(bf_hi(gw[j])) * bf_hi(uw[j]));
+        *reinterpret_cast<uint4 *>(out + r * ldo + c) = make_uint4(o[0], o[1], o[2], o[3]);
+    } else {
+        const float g = bf_lo(gate[r * ldi + c]);
+        out[r * ldo + c] = to_bf16(silu(g) * bf_lo(up[r * ldi + c]));
+    }
+}
+
+/* nearest-neighbour 2x upsampling of a channels-last image */
+template <int VEC>
+__global__ void __launch_bounds__(EW_THREADS)
+k_upsample2x(float *__restrict__ out, const float *__restrict__ in, int w, int c, size_t n) {
+    const size_t i = ((size_t)blockIdx.x * EW_THREADS + threadIdx.x) * VEC;
+    if (i >= n) return;
+    const int ch = (int)(i % c);
+    const size_t p = i / c;
+    const int x = (int)(p % (2 * (size_t)w)), y = (int)(p / (2 * (size_t)w));
+    const float *src = in + ((size_t)(y / 2) * w + x / 2) * c + ch;
+    if (VEC == 4) *reinterpret_cast<float4 *>(out + i) = *reinterpret_cast<const float4 *>(src);
+    else out[i] = *src;
+}
+
+/* ---------------------------------------------------------------- row normalisations */
+
+__device__ __forceinline__ float block_sum(float v, float *sh) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    const int wave = threadIdx.x >> 6;
+    __syncthreads();                                  /* sh may still be read from the previous reduction */
+    if ((threadIdx.x & 63) == 0) sh[wave] = v;
+    __syncthreads();
+    return sh[0] + sh[1] + sh[2] + sh[3];
+}
+
+enum NormKind { LAYER_NORM_MOD, RMS_NORM_MOD, RMS_NORM_RESIDUAL };
+
+/* One workgroup per row. CACHE: dim % 4 == 0, dim <= 4096, 16-byte aligned rows -> the row
+ * stays in registers (4 x float4 per thread). p0/p1 are (shift, scale) for LayerNorm,
+ * (w, scale) for RMSNorm, (w, gate) for the residual form; out_bf is unused by the latter. */
+template <int KIND, bool CACHE>
+__global__ void __launch_bounds__(ROW_THREADS)
+k_row_norm(uint16_t *__restrict__ out_bf, float *__restrict__ xres, const float *__restrict__ src,
+           const float *__restrict__ p0, const float *__restrict__ p1, int dim, float eps) {
+    __shared__ float sh[4];
+    const float *xr = src + (size_t)blockIdx.x * dim;
+    const int tid = threadIdx.x;
+    float4 keep[4];
+    const int nvec = dim >> 2;
+
+    float s = 0.0f;
+    if (CACHE) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int v = tid + j * ROW_THREADS;
+            keep[j] = v < nvec ? *reinterpret_cast<const float4 *>(xr + 4 * v) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (KIND == LAYER_NORM_MOD) s += (keep[j].x + keep[j].y) + (keep[j].z + keep[j].w);
+            else s += (keep[j].x * keep[j].x + keep[j].y * keep[j].y) + (keep[j].z * keep[j].z + keep[j].w * keep[j].w);
+        }
+    } else {
+        for (int i = tid; i < dim; i += ROW_THREADS) s += KIND == LAYER_NORM_MOD ? xr[i] : xr[i] * xr[i];
+    }
+    s = block_sum(s, sh);
+    float mean = 0.0f, inv;
+    if (KIND == LAYER_NORM_MOD) {
+        mean = s / (float)dim;
+        float v = 0.0f;
+        if (CACHE) {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (tid + j * ROW_THREADS < nvec) {
+                    const float a = keep[j].x - mean, b = keep[j].y - mean, c = keep[j].z - mean, d = keep[j].w - mean;
+                    v += (a * a + b * b) + (c * c + d * d);
+                }
+        } else {
+            for (int i = tid; i < dim; i += ROW_THREADS) { const float d = xr[i] - mean; v += d * d; }
+        }
+        inv = 1.0f / sqrtf(block_sum(v, sh) / (float)dim + eps);
+    } else {
+        inv = 1.0f / sqrtf(s / (float)dim + eps);
+    }
+
+    auto one = [&](float x, int i) -> float {
+        if (KIND == LAYER_NORM_MOD) {
+            float n = (x - mean) * inv;
+            if (p1) n *= 1.0f + p1[i];
+            if (p0) n += p0[i];
+            return n;
+        }
+        float v = x * inv * p0[i];
+        if (KIND == RMS_NORM_MOD) { if (p1) v *= 1.0f + p1[i]; return v; }
+        return (p1 ? tanhf(p1[i]) : 1.0f) * v;               /* residual form: the increment */
+    };
+    const size_t row_off = (size_t)blockIdx.x * dim;
+    if (CACHE) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int v = tid + j * ROW_THREADS;
+            if (v >= nvec) continue;
+            const float r0 = one(keep[j].x, 4 * v), r1 = one(keep[j].y, 4 * v + 1), r2 = one(keep[j].z, 4 * v + 2), r3 = one(keep[j].w, 4 * v + 3);
+            if (KIND == RMS_NORM_RESIDUAL) {
+                float4 t = *reinterpret_cast<float4 *>(xres + row_off + 4 * v);
+                t.x += r0; t.y += r1; t.z += r2; t.w += r3;
+                *reinterpret_cast<float4 *>(xres + row_off + 4 * v) = t;
+            } else {
+                *reinterpret_cast<uint2 *>(out_bf + row_off + 4 * v) = make_uint2(pack_bf16(r0, r1), pack_bf16(r2, r3));
+            }
+        }
+    } else {
+        for (int i = tid; i < dim; i += ROW_THREADS) {
+            const float r = one(xr[i], i);
+            if (KIND == RMS_NORM_RESIDUAL) xres[row_off + i] += r;
+            else out_bf[row_off + i] = to_bf16(r);
+        }
+    }
+}
+
+template <int KIND>
+int launch_row_norm(hipStream_t st, uint16_t *out_bf, float *xres, const float *src, const float *p0,
+                    const float *p1, int rows, int dim, float eps) {
+    if (rows <= 0 || dim <= 0) return 0;
+    const bool cache = dim % 4 == 0 && dim <= 4 * 4 * ROW_THREADS && al16(src) && al16(xres) && ((uintptr_t)out_bf & 7) == 0;
+    if (cache) hipLaunchKernelGGL((k_row_norm<KIND, true>), dim3(rows), dim3(ROW_THREADS), 0, st, out_bf, xres, src, p0, p1, dim, eps);
+    else hipLaunchKernelGGL((k_row_norm<KIND, false>), dim3(rows), dim3(ROW_THREADS), 0, st, out_bf, xres, src, p0, p1, dim, eps);
+    return (int)hipGetLastError();
+}
+
+/* ---------------------------------------------------------------- group norm */
+
+constexpr int GN_BLOCKS = 256;       /* partial sums per group */
+
+/* part[g * GN_BLOCKS + b] = sum over this block's share of group g of x (mean == NULL) or of
+ * (x - mean[g])^2. The group's hw * cg values are walked pixel by pixel, cg contiguous each. */
+__global__ void __launch_bounds__(ROW_THREADS)
+k_gn_partial(float *__restrict__ part, const float *__restrict__ in, const float *__restrict__ mean,
+             int hw, int c, int cg) {
+    __shared__ float sh[4];
+    const int g = blockIdx.x, b = blockIdx.y;
+    const size_t n = (size_t)hw * cg;
+    const size_t per_block = (n + GN_BLOCKS - 1) / GN_BLOCKS;
+    const size_t start = (size_t)b * per_block, end = start + per_block < n ? start + per_block : n;
+    const float m = mean ? mean[g] : 0.0f;
+    float s = 0.0f;
+    for (size_t i = start + threadIdx.x; i < end; i += ROW_THREADS) {
+        const float v = in[(i / cg) * c + (size_t)g * cg + i % cg];
+        s += mean ? (v - m) * (v - m) : v;
+    }
+    s = block_sum(s, sh);
+    if (threadIdx.x == 0) part[(size_t)g * GN_BLOCKS + b] = s;
+}
+
+/* stats[g] = mean (pass 0) or stats[groups + g] = 1 / sqrt(var + eps) (pass 1), in double */
+__global__ void k_gn_finalize(float *__restrict__ stats, const float *__restrict__ part, int groups,
+                              double count, float eps, int pass) {
+    const int g = blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= groups) return;
+    double s = 0.0;
+    for (int b = 0; b < GN_BLOCKS; b++) s += (double)part[(size_t)g * GN_BLOCKS + b];
+    if (pass == 0) stats[g] = (float)(s / count);
+    else stats[groups + g] = (float)(1.0 / sqrt(s / count + (double)eps));
+}
+
+template <int VEC>
+__global__ void __launch_bounds__(EW_THREADS)
+k_gn_apply(float *__restrict__ out, const float *__restrict__ in, const float *__restrict__ stats,
+           const float *__restrict__ gamma, const float *__restrict__ beta, int c, int cg, int groups,
+           int do_silu, size_t n) {
+    const size_t i = ((size_t)blockIdx.x * EW_THREADS + threadIdx.x) * VEC;
+    if (i >= n) return;
+    float v[VEC];
+    if (VEC == 4) *reinterpret_cast<float4 *>(v) = *reinterpret_cast<const float4 *>(in + i);
+    else v[0] = in[i];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+        const int ch = (int)((i + j) % c), g = ch / cg;
+        const float y = (v[j] - stats[g]) * stats[groups + g] * gamma[ch] + beta[ch];
+        v[j] = do_silu ? silu(y) : y;
+    }
+    if (VEC == 4) *reinterpret_cast<float4 *>(out + i) = *reinterpret_cast<float4 *>(v);
+    else out[i] = v[0];
+}
+
+}  // namespace
+
+extern "C" {
+
+int iris_hip_f32_to_bf16(void *stream, uint16_t *dst, const float *src, size_t n) {
+    if (!n) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    if (al16(dst) && al16(src) && n % 8 == 0)
+        hipLaunchKernelGGL(k_f32_to_bf16<8>, dim3(blocks_for(n, EW_THREADS * 8)), dim3(EW_THREADS), 0, st, dst, src, n);
+    else
+        hipLaunchKernelGGL(k_f32_to_bf16<1>, dim3(blocks_for(n, EW_THREADS)), dim3(EW_THREADS), 0, st, dst, src, n);
+    return (int)hipGetLastError();
+}
+
+int iris_hip_silu(void *stream, float *x, size_t n) { return launch_ew<OP_SILU>((hipStream_t)stream, x, nullptr, nullptr, 0, n); }
+int iris_hip_add(void *stream, float *x, const float *a, size_t n) { return launch_ew<OP_ADD>((hipStream_t)stream, x, a, nullptr, 0, n); }
+int iris_hip_add_bias(void *stream, float *y, const float *bias, int rows, int cols) {
+    return launch_ew<OP_ADD_ROW>((hipStream_t)stream, y, nullptr, bias, cols, (size_t)rows * cols);
+}
+int iris_hip_fill_rows(void *stream, float *out, const float *row, int rows, int dim) {
+    return launch_ew<OP_FILL_ROW>((hipStream_t)stream, out, nullptr, row, dim, (size_t)rows * dim);
+}
+/* x[r, c] += gate[c] * a[r, c], gate may be NULL */
+int iris_hip_residual(void *stream, float *x, const float *a, const float *gate, int rows, int dim) {
+    if (!gate) return launch_ew<OP_ADD>((hipStream_t)stream, x, a, nullptr, 0, (size_t)rows * dim);
+    return launch_ew<OP_MULADD_ROW>((hipStream_t)stream, x, a, gate, dim, (size_t)rows * dim);
+}
+
+int iris_hip_swiglu(void *stream, uint16_t *out, int ldo, const uint16_t *gate, const uint16_t *up, int ldi,
+                    int rows, int cols) {
+    const size_t n = (size_t)rows * cols;
+    if (!n) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    if (al16(out) && al16(gate) && al16(up) && cols % 8 == 0 && ldi % 8 == 0 && ldo % 8 == 0)
+        hipLaunchKernelGGL(k_swiglu<8>, dim3(blocks_for(n, EW_THREADS * 8)), dim3(EW_THREADS), 0, st, out, ldo, gate, up, ldi, cols, n);
+    else
+        hipLaunchKernelGGL(k_swiglu<1>, dim3(blocks_for(n, EW_THREADS)), dim3(EW_THREADS), 0, st, out, ldo, gate, up, ldi, cols, n);
+    return (int)hipGetLastError();
+}
+
+int iris_hip_upsample2x(void *stream, float *out, const float *in, int h, int width, int c) {
+    const size_t n = (size_t)4 * h * width * c;
+    if (!n) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    if (al16(out) && al16(in) && c % 4 == 0)
+        hipLaunchKernelGGL(k_upsample2x<4>, dim3(blocks_for(n, EW_THREADS * 4)), dim3(EW_THREADS), 0, st, out, in, width, c, n);
+    else
+        hipLaunchKernelGGL(k_upsample2x<1>, dim3(blocks_for(n, EW_THREADS)), dim3(EW_THREADS), 0, st, out, in, width, c, n);
+    return (int)hipGetLastError();
+}
+
+int iris_hip_layer_norm_mod(void *stream, uint16_t *out, const float *x, const float *shift, const float *scale,
+                            int rows, int dim, float eps) {
+    return launch_row_norm<LAYER_NORM_MOD>((hipStream_t)stream, out, nullptr, x, shift, scale, rows, dim, eps);
+}
+int iris_hip_rms_norm_mod(void *stream, uint16_t *out, const float *x, const float *w, const float *scale,
+                          int rows, int dim, float eps) {
+    return launch_row_norm<RMS_NORM_MOD>((hipStream_t)stream, out, nullptr, x, w, scale, rows, dim, eps);
+}
+int iris_hip_rms_norm_residual(void *stream, float *x, const float *a, const float *w, const float *gate,
+                               int rows, int dim, float eps) {
+    return launch_row_norm<RMS_NORM_RESIDUAL>((hipStream_t)stream, nullptr, x, a, w, gate, rows, dim, eps);
+}
+
+size_t iris_hip_group_norm_scratch_floats(int groups) { return (size_t)groups * GN_BLOCKS + 2 * (size_t)groups; }
+
+/* scratch: iris_hip_group_norm_scratch_floats(groups) floats of device memory */
+int iris_hip_group_norm(void *stream, float *scratch, float *out, const float *in, const float *gamma,
+                        const float *beta, int hw, int c, int groups, float eps, int do_silu) {
+    if (hw <= 0 || c <= 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    float *part = scratch, *stats = scratch + (size_t)groups * GN_BLOCKS;
+    const int cg = c / groups;
+    const double count = (double)hw * cg;
+    for (int pass = 0; pass < 2; pass++) {
+        hipLaunchKernelGGL(k_gn_partial, dim3(groups, GN_BLOCKS), dim3(ROW_THREADS), 0, st, part, in,
+                           pass ? stats : (const float *)nullptr, hw, c, cg);
+        hipLaunchKernelGGL(k_gn_finalize, dim3(blocks_for(groups, 64)), dim3(64), 0, st, stats, part, groups, count, eps, pass);
+    }
+    const size_t n = (size_t)hw * c;
+    if (al16(out) && al16(in) && c % 4 == 0)
+        hipLaunchKernelGGL(k_gn_apply<4>, dim3(blocks_for(n, EW_THREADS * 4)), dim3(EW_THREADS), 0, st, out, in, stats, gamma, beta, c, cg, groups, do_silu, n);
+    else
+        hipLaunchKernelGGL(k_gn_apply<1>, dim3(blocks_for(n, EW_THREADS)), dim3(EW_THREADS), 0, st, out, in, stats, gamma, beta, c, cg, groups, do_silu, n);
+    return (int)hipGetLastError();
+}
+
+}  // extern "C"

@@ -7,6 +7,7 @@
 #ifndef IRIS_KERNELS_HIP_H
 #define IRIS_KERNELS_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -45,6 +46,39 @@ int iris_hip_attention_generic(void *stream, uint16_t *out, int ldo, const uint1
                                const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
                                int seq_k, int heads, int kv_heads, int head_dim, float scale,
                                int causal, const int *key_mask);
+
+/* ---- elementwise and normalisation operators (ew_norm_ops.hip): any size and alignment,
+ * 16-byte accesses when the pointers and sizes allow ---- */
+int iris_hip_f32_to_bf16(void *stream, uint16_t *dst, const float *src, size_t n);
+int iris_hip_silu(void *stream, float *x, size_t n);
+int iris_hip_add(void *stream, float *x, const float *a, size_t n);
+int iris_hip_add_bias(void *stream, float *y, const float *bias, int rows, int cols);
+int iris_hip_fill_rows(void *stream, float *out, const float *row, int rows, int dim);
+int iris_hip_residual(void *stream, float *x, const float *a, const float *gate, int rows, int dim);
+int iris_hip_swiglu(void *stream, uint16_t *out, int ldo, const uint16_t *gate, const uint16_t *up,
+                    int ldi, int rows, int cols);
+int iris_hip_upsample2x(void *stream, float *out, const float *in, int h, int width, int c);
+int iris_hip_layer_norm_mod(void *stream, uint16_t *out, const float *x, const float *shift,
+                            const float *scale, int rows, int dim, float eps);
+int iris_hip_rms_norm_mod(void *stream, uint16_t *out, const float *x, const float *w,
+                          const float *scale, int rows, int dim, float eps);
+int iris_hip_rms_norm_residual(void *stream, float *x, const float *a, const float *w,
+                               const float *gate, int rows, int dim, float eps);
+/* group norm needs iris_hip_group_norm_scratch_floats(groups) floats of device scratch;
+ * requires c % groups == 0 */
+size_t iris_hip_group_norm_scratch_floats(int groups);
+int iris_hip_group_norm(void *stream, float *scratch, float *out, const float *in, const float *gamma,
+                        const float *beta, int hw, int c, int groups, float eps, int do_silu);
+
+/* ---- linear layers and convolution (gemm_conv_gfx950.hip) ---- */
+/* y[rows, out] = x[rows, in] @ W[out, in]^T, contiguous; MFMA kernel when in % 8 == 0 and
+ * x, W are 16-byte aligned, scalar kernel otherwise */
+int iris_hip_linear_f32(void *stream, float *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out);
+int iris_hip_linear_bf16(void *stream, uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out);
+/* convolution through bf16 patches in `scratch` (scratch_bytes >= 2 * k * k * cin) */
+int iris_hip_conv2d(void *stream, uint16_t *scratch, size_t scratch_bytes, float *out, const float *in,
+                    const uint16_t *w, const float *bias, int h, int width, int cin, int cout, int k,
+                    int stride, int pad_before, int pad_after);
 
 #ifdef __cplusplus
 }

@@ -26,6 +26,12 @@ static char g_name[640] = "none";
 static hipStream_t g_stream = NULL;
 static int g_last_error = 0;
 static const char *g_last_kernel = "none";
+/* private scratch, allocated on first use and kept until cleanup (as the reference backend
+ * does, iris_cuda.cu:149-173): convolution patches and group-norm partial sums */
+#define CONV_SCRATCH_BYTES ((size_t)256 << 20)
+static uint16_t *g_conv_scratch = NULL;
+static float *g_gn_scratch = NULL;
+static size_t g_gn_scratch_floats = 0;
 
 static void fail(int code, const char *what, const char *detail) {
     g_last_error = code ? code : -1;
@@ -79,6 +85,11 @@ int iris_dev_last_error(void) {
 void iris_dev_cleanup(void) {
     if (!g_ready) return;
     check(hipStreamSynchronize(g_stream), "sync");
+    if (g_conv_scratch) check(hipFree(g_conv_scratch), "free");
+    if (g_gn_scratch) check(hipFree(g_gn_scratch), "free");
+    g_conv_scratch = NULL;
+    g_gn_scratch = NULL;
+    g_gn_scratch_floats = 0;
     check(hipStreamDestroy(g_stream), "stream destroy");
     g_stream = NULL;
     g_ready = 0;
@@ -199,4 +210,122 @@ void iris_dev_attention(uint16_t *out, int ldo,
                                          kv_heads, head_dim, scale, causal != 0, key_mask);
     }
     if (err) check((hipError_t)err, "attention launch");
+}
+
+/* ---- the other operators: thin checked wrappers over the launchers ---- */
+
+#define LAUNCH(what, call)                                        \
+    do {                                                          \
+        if (!need_ready(what)) return;                            \
+        int err_ = (call);                                        \
+        if (err_) check((hipError_t)err_, what " launch");        \
+    } while (0)
+
+void iris_dev_f32_to_bf16(uint16_t *dst, const float *src, size_t n) {
+    LAUNCH("f32_to_bf16", iris_hip_f32_to_bf16(g_stream, dst, src, n));
+}
+
+void iris_dev_linear_f32(float *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out) {
+    if (rows <= 0 || out <= 0) return;
+    if (in <= 0) { fail(-1, "linear", "in must be positive"); return; }
+    LAUNCH("linear", iris_hip_linear_f32(g_stream, y, x, W, rows, in, out));
+}
+
+void iris_dev_linear_bf16(uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out) {
+    if (rows <= 0 || out <= 0) return;
+    if (in <= 0) { fail(-1, "linear", "in must be positive"); return; }
+    LAUNCH("linear", iris_hip_linear_bf16(g_stream, y, x, W, rows, in, out));
+}
+
+void iris_dev_layer_norm_mod(uint16_t *out, const float *x, const float *shift, const float *scale,
+                             int rows, int dim, float eps) {
+    LAUNCH("layer_norm_mod", iris_hip_layer_norm_mod(g_stream, out, x, shift, scale, rows, dim, eps));
+}
+
+void iris_dev_rms_norm(uint16_t *out, const float *x, const float *w, int rows, int dim, float eps) {
+    LAUNCH("rms_norm", iris_hip_rms_norm_mod(g_stream, out, x, w, NULL, rows, dim, eps));
+}
+
+void iris_dev_rms_norm_mod(uint16_t *out, const float *x, const float *w, const float *scale,
+                           int rows, int dim, float eps) {
+    LAUNCH("rms_norm_mod", iris_hip_rms_norm_mod(g_stream, out, x, w, scale, rows, dim, eps));
+}
+
+void iris_dev_rms_norm_residual(float *x, const float *a, const float *w, const float *gate,
+                                int rows, int dim, float eps) {
+    LAUNCH("rms_norm_residual", iris_hip_rms_norm_residual(g_stream, x, a, w, gate, rows, dim, eps));
+}
+
+void iris_dev_swiglu(uint16_t *out, int ldo, const uint16_t *gate, const uint16_t *up, int ldi,
+                     int rows, int cols) {
+    if (rows <= 0 || cols <= 0) return;
+    LAUNCH("swiglu", iris_hip_swiglu(g_stream, out, ldo, gate, up, ldi, rows, cols));
+}
+
+void iris_dev_residual(float *x, const float *a, const float *gate, int rows, int dim) {
+    if (rows <= 0 || dim <= 0) return;
+    LAUNCH("residual", iris_hip_residual(g_stream, x, a, gate, rows, dim));
+}
+
+void iris_dev_silu(float *x, size_t n) { LAUNCH("silu", iris_hip_silu(g_stream, x, n)); }
+void iris_dev_add(float *x, const float *a, size_t n) { LAUNCH("add", iris_hip_add(g_stream, x, a, n)); }
+
+void iris_dev_add_bias(float *y, const float *bias, int rows, int cols) {
+    if (rows <= 0 || cols <= 0) return;
+    LAUNCH("add_bias", iris_hip_add_bias(g_stream, y, bias, rows, cols));
+}
+
+void iris_dev_fill_rows(float *out, const float *row, int rows, int dim) {
+    if (rows <= 0 || dim <= 0) return;
+    LAUNCH("fill_rows", iris_hip_fill_rows(g_stream, out, row, rows, dim));
+}
+
+void iris_dev_conv2d(float *out, const float *in, const uint16_t *w, const float *bias,
+                     int h, int width, int cin, int cout, int k, int stride,
+                     int pad_before, int pad_after) {
+    if (!need_ready("conv2d")) return;
+    if (h <= 0 || width <= 0 || cin <= 0 || cout <= 0 || k <= 0 || stride <= 0 || pad_before < 0 || pad_after < 0 ||
+        (size_t)k * k * cin * sizeof(uint16_t) > CONV_SCRATCH_BYTES) {
+        fail(-1, "conv2d", "bad shape");
+        return;
+    }
+    if (!g_conv_scratch && hipMalloc((void **)&g_conv_scratch, CONV_SCRATCH_BYTES) != hipSuccess) {
+        (void)hipGetLastError();
+        g_conv_scratch = NULL;
+        fail(-1, "conv2d", "scratch allocation failed");
+        return;
+    }
+    int err = iris_hip_conv2d(g_stream, g_conv_scratch, CONV_SCRATCH_BYTES, out, in, w, bias, h, width, cin, cout,
+                              k, stride, pad_before, pad_after);
+    if (err) check((hipError_t)err, "conv2d launch");
+}
+
+void iris_dev_group_norm(float *out, const float *in, const float *gamma, const float *beta,
+                         int hw, int c, int groups, float eps, int silu) {
+    if (!need_ready("group_norm")) return;
+    if (hw <= 0 || c <= 0) return;
+    if (groups <= 0 || c % groups != 0) { fail(-1, "group_norm", "need c % groups == 0"); return; }
+    size_t need = iris_hip_group_norm_scratch_floats(groups);
+    if (need > g_gn_scratch_floats) {
+        if (g_gn_scratch) {
+            check(hipStreamSynchronize(g_stream), "sync");
+            check(hipFree(g_gn_scratch), "free");
+        }
+        g_gn_scratch = NULL;
+        g_gn_scratch_floats = 0;
+        if (hipMalloc((void **)&g_gn_scratch, need * sizeof(float)) != hipSuccess) {
+            (void)hipGetLastError();
+            g_gn_scratch = NULL;
+            fail(-1, "group_norm", "scratch allocation failed");
+            return;
+        }
+        g_gn_scratch_floats = need;
+    }
+    int err = iris_hip_group_norm(g_stream, g_gn_scratch, out, in, gamma, beta, hw, c, groups, eps, silu != 0);
+    if (err) check((hipError_t)err, "group_norm launch");
+}
+
+void iris_dev_upsample2x(float *out, const float *in, int h, int width, int c) {
+    if (h <= 0 || width <= 0 || c <= 0) return;
+    LAUNCH("upsample2x", iris_hip_upsample2x(g_stream, out, in, h, width, c));
 }
