@@ -5,10 +5,12 @@
  * accesses per lane where the pointers and sizes allow it, a scalar form of
  * the same kernel otherwise.
  *
- * Row normalisations use one workgroup (256 threads) per row and keep the
- * row in registers between the statistics and the write (rows up to 4096
- * floats; longer rows are read again, from cache). Statistics follow the
- * reference: LayerNorm takes the mean first and the variance about it.
+ * Row normalisations use one wave per row (four rows per workgroup, no LDS,
+ * no barrier) and keep the row in registers between the statistics and the
+ * write (rows up to 4096 floats; longer rows are read again, from cache).
+ * Statistics follow the reference: LayerNorm takes the mean first and the
+ * variance about it. Group norm does the same in two passes over the image
+ * with coalesced per-pixel reads and per-group partial sums.
  */
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -129,9 +131,14 @@ k_upsample2x(float *__restrict__ out, const float *__restrict__ in, int w, int c
 
 /* ---------------------------------------------------------------- row normalisations */
 
-__device__ __forceinline__ float block_sum(float v, float *sh) {
+__device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ float block_sum(float v, float *sh) {
+    v = wave_sum(v);
     const int wave = threadIdx.x >> 6;
     __syncthreads();                                  /* sh may still be read from the previous reduction */
     if ((threadIdx.x & 63) == 0) sh[wave] = v;
@@ -140,81 +147,100 @@ __device__ __forceinline__ float block_sum(float v, float *sh) {
 }
 
 enum NormKind { LAYER_NORM_MOD, RMS_NORM_MOD, RMS_NORM_RESIDUAL };
+constexpr int ROW_VECS = 16;          /* float4 per lane kept in registers: rows up to 4096 floats */
 
-/* One workgroup per row. CACHE: dim % 4 == 0, dim <= 4096, 16-byte aligned rows -> the row
- * stays in registers (4 x float4 per thread). p0/p1 are (shift, scale) for LayerNorm,
+/* One WAVE per row, four rows per workgroup: no LDS, no barrier. CACHE: dim % 4 == 0,
+ * dim <= 4096, 16-byte aligned rows -> the row stays in registers between the statistics
+ * and the write; otherwise it is read again. p0/p1 are (shift, scale) for LayerNorm,
  * (w, scale) for RMSNorm, (w, gate) for the residual form; out_bf is unused by the latter. */
 template <int KIND, bool CACHE>
 __global__ void __launch_bounds__(ROW_THREADS)
 k_row_norm(uint16_t *__restrict__ out_bf, float *__restrict__ xres, const float *__restrict__ src,
-           const float *__restrict__ p0, const float *__restrict__ p1, int dim, float eps) {
-    __shared__ float sh[4];
-    const float *xr = src + (size_t)blockIdx.x * dim;
-    const int tid = threadIdx.x;
-    float4 keep[4];
+           const float *__restrict__ p0, const float *__restrict__ p1, int rows, int dim, float eps) {
+    const int row = blockIdx.x * (ROW_THREADS / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const float *xr = src + (size_t)row * dim;
+    float4 keep[ROW_VECS];
     const int nvec = dim >> 2;
 
     float s = 0.0f;
     if (CACHE) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int v = tid + j * ROW_THREADS;
+        for (int j = 0; j < ROW_VECS; j++) {
+            const int v = lane + j * 64;
             keep[j] = v < nvec ? *reinterpret_cast<const float4 *>(xr + 4 * v) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if (KIND == LAYER_NORM_MOD) s += (keep[j].x + keep[j].y) + (keep[j].z + keep[j].w);
             else s += (keep[j].x * keep[j].x + keep[j].y * keep[j].y) + (keep[j].z * keep[j].z + keep[j].w * keep[j].w);
         }
     } else {
-        for (int i = tid; i < dim; i += ROW_THREADS) s += KIND == LAYER_NORM_MOD ? xr[i] : xr[i] * xr[i];
+        for (int i = lane; i < dim; i += 64) s += KIND == LAYER_NORM_MOD ? xr[i] : xr[i] * xr[i];
     }
-    s = block_sum(s, sh);
+    s = wave_sum(s);
     float mean = 0.0f, inv;
     if (KIND == LAYER_NORM_MOD) {
         mean = s / (float)dim;
         float v = 0.0f;
         if (CACHE) {
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                if (tid + j * ROW_THREADS < nvec) {
+            for (int j = 0; j < ROW_VECS; j++)
+                if (lane + j * 64 < nvec) {
                     const float a = keep[j].x - mean, b = keep[j].y - mean, c = keep[j].z - mean, d = keep[j].w - mean;
                     v += (a * a + b * b) + (c * c + d * d);
                 }
         } else {
-            for (int i = tid; i < dim; i += ROW_THREADS) { const float d = xr[i] - mean; v += d * d; }
+            for (int i = lane; i < dim; i += 64) { const float d = xr[i] - mean; v += d * d; }
         }
-        inv = 1.0f / sqrtf(block_sum(v, sh) / (float)dim + eps);
+        inv = 1.0f / sqrtf(wave_sum(v) / (float)dim + eps);
     } else {
         inv = 1.0f / sqrtf(s / (float)dim + eps);
     }
 
-    auto one = [&](float x, int i) -> float {
-        if (KIND == LAYER_NORM_MOD) {
-            float n = (x - mean) * inv;
-            if (p1) n *= 1.0f + p1[i];
-            if (p0) n += p0[i];
-            return n;
-        }
-        float v = x * inv * p0[i];
-        if (KIND == RMS_NORM_MOD) { if (p1) v *= 1.0f + p1[i]; return v; }
-        return (p1 ? tanhf(p1[i]) : 1.0f) * v;               /* residual form: the increment */
-    };
-    const size_t row_off = (size_t)blockIdx.x * dim;
+    const size_t row_off = (size_t)row * dim;
     if (CACHE) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int v = tid + j * ROW_THREADS;
+        for (int j = 0; j < ROW_VECS; j++) {
+            const int v = lane + j * 64;
             if (v >= nvec) continue;
-            const float r0 = one(keep[j].x, 4 * v), r1 = one(keep[j].y, 4 * v + 1), r2 = one(keep[j].z, 4 * v + 2), r3 = one(keep[j].w, 4 * v + 3);
+            const float xin[4] = {keep[j].x, keep[j].y, keep[j].z, keep[j].w};
+            float4 a = *reinterpret_cast<const float4 *>(KIND == LAYER_NORM_MOD ? (p1 ? p1 : xr) + 4 * v : p0 + 4 * v);   /* scale | w */
+            float4 b = *reinterpret_cast<const float4 *>((KIND == LAYER_NORM_MOD ? (p0 ? p0 : xr) : (p1 ? p1 : xr)) + 4 * v);   /* shift | scale/gate */
+            const float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+            float r[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                if (KIND == LAYER_NORM_MOD) {
+                    float n = (xin[e] - mean) * inv;
+                    if (p1) n *= 1.0f + av[e];
+                    if (p0) n += bv[e];
+                    r[e] = n;
+                } else {
+                    float t = xin[e] * inv * av[e];
+                    if (KIND == RMS_NORM_MOD) { if (p1) t *= 1.0f + bv[e]; }
+                    else t *= p1 ? tanhf(bv[e]) : 1.0f;
+                    r[e] = t;
+                }
+            }
             if (KIND == RMS_NORM_RESIDUAL) {
                 float4 t = *reinterpret_cast<float4 *>(xres + row_off + 4 * v);
-                t.x += r0; t.y += r1; t.z += r2; t.w += r3;
+                t.x += r[0]; t.y += r[1]; t.z += r[2]; t.w += r[3];
                 *reinterpret_cast<float4 *>(xres + row_off + 4 * v) = t;
             } else {
-                *reinterpret_cast<uint2 *>(out_bf + row_off + 4 * v) = make_uint2(pack_bf16(r0, r1), pack_bf16(r2, r3));
+                *reinterpret_cast<uint2 *>(out_bf + row_off + 4 * v) = make_uint2(pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]));
             }
         }
     } else {
-        for (int i = tid; i < dim; i += ROW_THREADS) {
-            const float r = one(xr[i], i);
+        for (int i = lane; i < dim; i += 64) {
+            float r;
+            if (KIND == LAYER_NORM_MOD) {
+                r = (xr[i] - mean) * inv;
+                if (p1) r *= 1.0f + p1[i];
+                if (p0) r += p0[i];
+            } else {
+                r = xr[i] * inv * p0[i];
+                if (KIND == RMS_NORM_MOD) { if (p1) r *= 1.0f + p1[i]; }
+                else r *= p1 ? tanhf(p1[i]) : 1.0f;
+            }
             if (KIND == RMS_NORM_RESIDUAL) xres[row_off + i] += r;
             else out_bf[row_off + i] = to_bf16(r);
         }
@@ -225,9 +251,11 @@ template <int KIND>
 int launch_row_norm(hipStream_t st, uint16_t *out_bf, float *xres, const float *src, const float *p0,
                     const float *p1, int rows, int dim, float eps) {
     if (rows <= 0 || dim <= 0) return 0;
-    const bool cache = dim % 4 == 0 && dim <= 4 * 4 * ROW_THREADS && al16(src) && al16(xres) && ((uintptr_t)out_bf & 7) == 0;
-    if (cache) hipLaunchKernelGGL((k_row_norm<KIND, true>), dim3(rows), dim3(ROW_THREADS), 0, st, out_bf, xres, src, p0, p1, dim, eps);
-    else hipLaunchKernelGGL((k_row_norm<KIND, false>), dim3(rows), dim3(ROW_THREADS), 0, st, out_bf, xres, src, p0, p1, dim, eps);
+    const bool cache = dim % 4 == 0 && dim <= 4 * 64 * ROW_VECS && al16(src) && al16(xres) && al16(p0) && al16(p1) &&
+                       ((uintptr_t)out_bf & 7) == 0;
+    const unsigned blocks = (unsigned)((rows + ROW_THREADS / 64 - 1) / (ROW_THREADS / 64));
+    if (cache) hipLaunchKernelGGL((k_row_norm<KIND, true>), dim3(blocks), dim3(ROW_THREADS), 0, st, out_bf, xres, src, p0, p1, rows, dim, eps);
+    else hipLaunchKernelGGL((k_row_norm<KIND, false>), dim3(blocks), dim3(ROW_THREADS), 0, st, out_bf, xres, src, p0, p1, rows, dim, eps);
     return (int)hipGetLastError();
 }
 
@@ -235,8 +263,37 @@ int launch_row_norm(hipStream_t st, uint16_t *out_bf, float *xres, const float *
 
 constexpr int GN_BLOCKS = 256;       /* partial sums per group */
 
-/* part[g * GN_BLOCKS + b] = sum over this block's share of group g of x (mean == NULL) or of
- * (x - mean[g])^2. The group's hw * cg values are walked pixel by pixel, cg contiguous each. */
+/* part[g * GN_BLOCKS + b] = sum over block b's pixels of group g of x (mean == NULL) or of
+ * (x - mean[g])^2. Coalesced form: needs c % 4 == 0, cg % 4 == 0 and (c / 4) dividing 256;
+ * a thread keeps one quad of channels, the workgroup walks 256 / (c / 4) pixels per step. */
+__global__ void __launch_bounds__(ROW_THREADS)
+k_gn_partial_rows(float *__restrict__ part, const float *__restrict__ in, const float *__restrict__ mean,
+                  int hw, int c, int cg) {
+    __shared__ float sh[ROW_THREADS];
+    const int quads = c >> 2, ppi = ROW_THREADS / quads;      /* pixels per iteration */
+    const int q = threadIdx.x % quads, sub = threadIdx.x / quads;
+    const int g = (4 * q) / cg;
+    const float m = mean ? mean[g] : 0.0f;
+    const int per_block = (hw + GN_BLOCKS - 1) / GN_BLOCKS;
+    const int start = blockIdx.x * per_block, end = min(start + per_block, hw);
+    float s = 0.0f;
+    for (int p = start + sub; p < end; p += ppi) {
+        const float4 v = *reinterpret_cast<const float4 *>(in + (size_t)p * c + 4 * q);
+        if (mean) s += ((v.x - m) * (v.x - m) + (v.y - m) * (v.y - m)) + ((v.z - m) * (v.z - m) + (v.w - m) * (v.w - m));
+        else s += (v.x + v.y) + (v.z + v.w);
+    }
+    sh[threadIdx.x] = s;
+    __syncthreads();
+    const int groups = c / cg, qpg = cg >> 2;
+    if ((int)threadIdx.x < groups) {
+        float t = 0.0f;
+        for (int sb = 0; sb < ppi; sb++)
+            for (int j = 0; j < qpg; j++) t += sh[sb * quads + threadIdx.x * qpg + j];
+        part[(size_t)threadIdx.x * GN_BLOCKS + blockIdx.x] = t;
+    }
+}
+
+/* Any shape: one workgroup per (group, block), strided reads. */
 __global__ void __launch_bounds__(ROW_THREADS)
 k_gn_partial(float *__restrict__ part, const float *__restrict__ in, const float *__restrict__ mean,
              int hw, int c, int cg) {
@@ -360,9 +417,14 @@ int iris_hip_group_norm(void *stream, float *scratch, float *out, const float *i
     float *part = scratch, *stats = scratch + (size_t)groups * GN_BLOCKS;
     const int cg = c / groups;
     const double count = (double)hw * cg;
+    const bool rows_form = c % 4 == 0 && cg % 4 == 0 && c / 4 <= ROW_THREADS && ROW_THREADS % (c / 4) == 0 && al16(in);
     for (int pass = 0; pass < 2; pass++) {
-        hipLaunchKernelGGL(k_gn_partial, dim3(groups, GN_BLOCKS), dim3(ROW_THREADS), 0, st, part, in,
-                           pass ? stats : (const float *)nullptr, hw, c, cg);
+        if (rows_form)
+            hipLaunchKernelGGL(k_gn_partial_rows, dim3(GN_BLOCKS), dim3(ROW_THREADS), 0, st, part, in,
+                               pass ? stats : (const float *)nullptr, hw, c, cg);
+        else
+            hipLaunchKernelGGL(k_gn_partial, dim3(groups, GN_BLOCKS), dim3(ROW_THREADS), 0, st, part, in,
+                               pass ? stats : (const float *)nullptr, hw, c, cg);
         hipLaunchKernelGGL(k_gn_finalize, dim3(blocks_for(groups, 64)), dim3(64), 0, st, stats, part, groups, count, eps, pass);
     }
     const size_t n = (size_t)hw * c;

@@ -65,3 +65,21 @@ def test_product_does_not_link_the_oracle(lib):
             if f.endswith((".c", ".h", ".hip", ".py")):
                 src = open(os.path.join(root, f)).read()
                 assert "import oracle" not in src and "iris_oracle.h" not in src and "orc_" not in src, f
+
+
+def test_unmodified_reference_links_against_this_backend(lib):
+    """The reference's own host program (models, sampler, CLI, main), compiled with its device path
+    enabled, links against this library in place of the reference's GPU backend: every iris_dev_*
+    symbol it uses is exported here. Link check only (built where the reference tree exists)."""
+    import subprocess
+    if not os.path.isdir("/root/reference"):
+        pytest.skip("reference tree not present on this machine")
+    subprocess.check_call(["make", "-s", "-C", os.path.join(ROOT, "oracle"), "linkcheck"])
+    exe = os.path.join(ROOT, "oracle", "_ref", "iris_linked_to_this_backend")
+    undefined = subprocess.run(["nm", "-D", "--undefined-only", exe], capture_output=True, text=True, check=True).stdout
+    used = sorted({line.split()[-1] for line in undefined.splitlines() if " iris_dev_" in line})
+    assert len(used) >= 28
+    import iris_c_amd
+    assert set(used) <= set(iris_c_amd.ABI), sorted(set(used) - set(iris_c_amd.ABI))
+    ldd = subprocess.run(["ldd", exe], capture_output=True, text=True, check=True).stdout
+    assert "libiris_dev.so" in ldd and "not found" not in ldd
