@@ -12,7 +12,8 @@ Prints ONE JSON line. `value` is attention TFLOP/s over the whole step
 (algorithmic attention FLOPs / wall time of the triple). `roofline` is the
 attention kernel alone, timed with HIP events on the library's stream.
 `norm_rope` reports the bandwidth-bound kernel the same way. `shapes` lists
-latency / TFLOP/s / GB/s for every benchmark configuration. `cpu_baseline`
+latency / TFLOP/s / GB/s for every benchmark configuration, `other_ops` the
+other device operators at this configuration's shapes. `cpu_baseline`
 times the reference's BLAS-build CPU structure on this host's cores.
 """
 import argparse
@@ -196,6 +197,45 @@ def per_launch_times(hip, stream, fn, reps):
     for i, (a, b) in enumerate(evs):
         hip.record(a, stream); fn(i); hip.record(b, stream)
     return [hip.elapsed_ms(a, b) for a, b in evs]
+
+
+# ----------------------------------------------------------------------------- the other operators
+def other_ops(dev, hip, stream, rng):
+    """Latency of the other device operators at the shapes a transformer block of the bench configuration
+    uses (4608 tokens, width 3072): linear layers in TFLOP/s, one-pass kernels in GB/s (bytes read + written)."""
+    lib = dev.lib
+    rows, dim = 4608, 3072
+    res = []
+
+    def timed(fn, reps=10):
+        fn(0); lib.iris_dev_sync(); dev.check()
+        return min(event_time(hip, stream, fn, reps) for _ in range(3))
+
+    x = dev.to_device(to_bf16(rng.standard_normal((rows, 12288), dtype=np.float32)))
+    W = dev.to_device(to_bf16(rng.standard_normal((27648 * 3072,), dtype=np.float32) * 0.02))
+    y = lib.iris_dev_alloc(rows * 27648 * 4)
+    for k, n in ((3072, 9216), (3072, 3072), (3072, 18432), (9216, 3072), (3072, 27648), (12288, 3072)):
+        for name, fn in (("linear_f32", lib.iris_dev_linear_f32), ("linear_bf16", lib.iris_dev_linear_bf16)):
+            ms = timed(lambda i: fn(y, x, W, rows, k, n), 5)
+            res.append({"op": name, "shape": f"{rows}x{k}->{n}", "us": round(ms * 1e3, 1),
+                        "tflops": round(2 * rows * k * n / ms / 1e9, 1)})
+    xf, af = _vp(y), _vp(y + rows * dim * 4)
+    w1 = dev.to_device(np.ones(dim, np.float32))
+    ob = _vp(x)
+    n = rows * dim
+    one_pass = [("layer_norm_mod", lambda i: lib.iris_dev_layer_norm_mod(ob, xf, w1, w1, rows, dim, 1e-6), 6 * n),
+                ("rms_norm", lambda i: lib.iris_dev_rms_norm(ob, xf, w1, rows, dim, 1e-6), 6 * n),
+                ("rms_norm_residual", lambda i: lib.iris_dev_rms_norm_residual(xf, af, w1, w1, rows, dim, 1e-6), 12 * n),
+                ("residual", lambda i: lib.iris_dev_residual(xf, af, w1, rows, dim), 12 * n),
+                ("f32_to_bf16", lambda i: lib.iris_dev_f32_to_bf16(ob, xf, n), 6 * n),
+                ("swiglu 4608x9216", lambda i: lib.iris_dev_swiglu(ob, 9216, _vp(y), _vp(y + 2 * 9216), 18432, rows, 9216), 6 * rows * 9216)]
+    for name, fn, nbytes in one_pass:
+        ms = timed(fn, 20)
+        res.append({"op": name, "shape": f"{rows}x{dim}" if "swiglu" not in name else "", "us": round(ms * 1e3, 1),
+                    "gbps": round(nbytes / ms / 1e6, 0)})
+    for p in (x, W, y, w1):
+        lib.iris_dev_free(p)
+    return res
 
 
 # ----------------------------------------------------------------------------- machine ceilings
@@ -391,6 +431,8 @@ def main():
             r.free()
         out["shapes"] = shapes
 
+    if not args.no_shapes:
+        out["other_ops"] = other_ops(dev, hip, stream, rng)
     if not args.no_machine:
         out["machine"] = machine_ceilings(dev, hip, stream)
         # The ABI takes device pointers, so `value` has no host transfer in it. For a caller that had the

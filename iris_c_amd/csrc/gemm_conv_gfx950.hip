@@ -11,7 +11,7 @@
  * the 16x16 accumulator a lane then holds four consecutive n of one output row m,
  * a single 16-byte (f32) or 8-byte (bf16) store.
  *
- * Workgroup = 4 waves (2 x 2), tile 128 (m) x 128 (n), K in steps of 64; a wave owns
+ * Workgroup = WM x WN waves (2 x 2 in use), tile 128 (m) x 128 (n), K in steps of 64; a wave owns
  * 64 x 64 = 4 x 4 accumulator blocks and reads 8 operands from LDS per 16 MFMAs. One
  * LDS stage of [W tile | x tile], rows padded to 160 B so that the 16 lanes the LDS
  * serves together on a 128-bit read fall in distinct bank windows; the next K tile
@@ -39,9 +39,8 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int TM = 128, TN = 128, TK = 64;
+constexpr int TK = 64;
 constexpr int LS = TK + 16;            /* LDS row stride in elements (160 B) */
-constexpr int THREADS = 256;
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     f32x2 p = {lo, hi};
@@ -61,10 +60,14 @@ __device__ __forceinline__ void store4(uint16_t *p, f32x4 v, int n_left) {
     for (int r = 0; r < 4 && r < n_left; r++) p[r] = (uint16_t)(pack_bf16(v[r], 0.0f) & 0xffffu);
 }
 
-template <typename OUT>
-__global__ void __launch_bounds__(THREADS, 2)
+/* WM x WN waves of 64 x 64 outputs each: tile (64 WM) x (64 WN). */
+template <typename OUT, int WM, int WN>
+__global__ void __launch_bounds__(64 * WM * WN, 2)
 k_gemm_bf16(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *__restrict__ W,
             int M, int N, int K, int tiles_m) {
+    constexpr int TM = 64 * WM, TN = 64 * WN, THREADS = 64 * WM * WN;
+    constexpr int RPP = THREADS / 8;                 /* rows covered by one pass of the workgroup */
+    constexpr int NW = TN / RPP, NX = TM / RPP;      /* 16 B chunks of W and of x per thread and K tile */
     __shared__ __align__(16) uint16_t lds[(TN + TM) * LS];
     uint16_t *Ws = lds, *Xs = lds + TN * LS;
 
@@ -72,31 +75,28 @@ k_gemm_bf16(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t 
     const int m0 = bm * TM, n0 = bn * TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, lg = lane >> 4;
-    const int wm = wave & 1, wn = wave >> 1;
+    const int wm = wave % WM, wn = wave / WM;
 
-    /* staging: this thread moves 16 B chunk (tid % 8) of rows tid / 8 + 32 c of both tiles */
+    /* staging: this thread moves 16 B chunk (tid % 8) of rows tid / 8 + RPP c of both tiles */
     const int srow = tid >> 3, scol = (tid & 7) * 8;
-    const uint16_t *wsrc[4], *xsrc[4];
+    const uint16_t *wsrc[NW], *xsrc[NX];
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
-        wsrc[c] = W + (size_t)min(n0 + srow + 32 * c, N - 1) * K + scol;
-        xsrc[c] = x + (size_t)min(m0 + srow + 32 * c, M - 1) * K + scol;
-    }
-    u32x4 wreg[4], xreg[4];
+    for (int c = 0; c < NW; c++) wsrc[c] = W + (size_t)min(n0 + srow + RPP * c, N - 1) * K + scol;
+#pragma unroll
+    for (int c = 0; c < NX; c++) xsrc[c] = x + (size_t)min(m0 + srow + RPP * c, M - 1) * K + scol;
+    u32x4 wreg[NW], xreg[NX];
     auto fetch = [&](int k0) {
         const bool inside = k0 + scol < K;                 /* K % 8 == 0: a chunk is inside or outside */
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            wreg[c] = inside ? *reinterpret_cast<const u32x4 *>(wsrc[c] + k0) : u32x4{0, 0, 0, 0};
-            xreg[c] = inside ? *reinterpret_cast<const u32x4 *>(xsrc[c] + k0) : u32x4{0, 0, 0, 0};
-        }
+        for (int c = 0; c < NW; c++) wreg[c] = inside ? *reinterpret_cast<const u32x4 *>(wsrc[c] + k0) : u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int c = 0; c < NX; c++) xreg[c] = inside ? *reinterpret_cast<const u32x4 *>(xsrc[c] + k0) : u32x4{0, 0, 0, 0};
     };
     auto store = [&]() {
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            *reinterpret_cast<u32x4 *>(&Ws[(srow + 32 * c) * LS + scol]) = wreg[c];
-            *reinterpret_cast<u32x4 *>(&Xs[(srow + 32 * c) * LS + scol]) = xreg[c];
-        }
+        for (int c = 0; c < NW; c++) *reinterpret_cast<u32x4 *>(&Ws[(srow + RPP * c) * LS + scol]) = wreg[c];
+#pragma unroll
+        for (int c = 0; c < NX; c++) *reinterpret_cast<u32x4 *>(&Xs[(srow + RPP * c) * LS + scol]) = xreg[c];
     };
 
     f32x4 acc[4][4];
@@ -166,8 +166,11 @@ template <typename OUT>
 int gemm(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, int N, int K) {
     if (M <= 0 || N <= 0) return 0;
     if (K > 0 && K % 8 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)W & 15) == 0) {
+        /* 2 x 2 waves (128 x 128 tiles) measured best on the transformer shapes: 4 x 2 and 2 x 4 are
+         * 5-8 % slower on the wide projections, 4 x 1 and 2 x 1 15-30 % slower. */
+        constexpr int WM = 2, WN = 2, TM = 64 * WM, TN = 64 * WN;
         const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
-        hipLaunchKernelGGL(k_gemm_bf16<OUT>, dim3((unsigned)tiles_m * tiles_n), dim3(THREADS), 0, st, y, x, W, M, N, K, tiles_m);
+        hipLaunchKernelGGL((k_gemm_bf16<OUT, WM, WN>), dim3((unsigned)tiles_m * tiles_n), dim3(64 * WM * WN), 0, st, y, x, W, M, N, K, tiles_m);
     } else {
         const size_t n = (size_t)M * N;
         hipLaunchKernelGGL(k_gemm_scalar<OUT>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, y, x, W, M, N, K);
