@@ -31,8 +31,8 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 matrix peak (vendor figure)
 PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E peak
 # HBM bytes one C2 attention launch moves, from the FETCH_SIZE and WRITE_SIZE hardware counters scaled by a
-# 1 GiB copy kernel (profiles/k_fa_fwd_hd128__c2__hbm_traffic.txt): 104.0 MB read + 28.3 MB written.
-C2_ATTENTION_HBM_TRAFFIC = 132_353_000
+# 1 GiB copy kernel (profiles/k_fa_fwd_hd128__c2__hbm_traffic.txt): 103.9 MB read + 28.3 MB written.
+C2_ATTENTION_HBM_TRAFFIC = 132_174_000
 
 _vp = C.c_void_p
 
