@@ -71,6 +71,37 @@ def main():
                                          inputs(132, kv * hd, hidden) / 5, inputs(133, kv * hd, hidden) / 5,
                                          1 + 0.02 * inputs(134, hd), 1 + 0.02 * inputs(135, hd), qmask, heads, kv, hd)
     g["qwen3_attention"], g["qwen3_q"], g["qwen3_k"] = attn, rq, rk
+    # --- the other device operators: outputs of the reference's CPU twins (NCHW there; the test transposes)
+    import ctypes as C
+    P = lambda a: a.ctypes.data_as(C.c_void_p)
+    xl = oracle.bf16_to_f32(oracle.f32_to_bf16(inputs(140, 7, 96)))
+    Wl = oracle.f32_to_bf16(inputs(141, 33, 96) * 0.1)
+    yl = np.empty((7, 33), np.float32)
+    refi.lib.iris_linear_nobias_bf16(P(yl), P(np.ascontiguousarray(xl)), P(Wl), C.c_int(7), C.c_int(96), C.c_int(33))
+    g["ops_linear"] = yl
+    xs = inputs(142, 500) * 3
+    ys = xs.copy()
+    refi.lib.iris_silu(P(ys), C.c_int(ys.size))
+    g["ops_silu"] = ys
+    h, w, cin, cout, k = 6, 5, 8, 4, 3
+    img = oracle.bf16_to_f32(oracle.f32_to_bf16(inputs(143, h * w, cin)))
+    wt = oracle.bf16_to_f32(oracle.f32_to_bf16(inputs(144, cout, k * k * cin) * 0.2))
+    bias = inputs(145, cout)
+    x_nchw = np.ascontiguousarray(img.reshape(h, w, cin).transpose(2, 0, 1))
+    w_nchw = np.ascontiguousarray(wt.reshape(cout, k, k, cin).transpose(0, 3, 1, 2))
+    yc = np.empty((cout, h, w), np.float32)
+    refi.lib.iris_conv2d(P(yc), P(x_nchw), P(w_nchw), P(bias), C.c_int(1), C.c_int(cin), C.c_int(cout), C.c_int(h), C.c_int(w),
+                         C.c_int(k), C.c_int(k), C.c_int(1), C.c_int(1))
+    g["ops_conv2d"] = np.ascontiguousarray(yc.transpose(1, 2, 0).reshape(h * w, cout))
+    gimg, gamma, beta = inputs(146, 30, 16) * 2 + 0.5, 1 + 0.1 * inputs(147, 16), 0.1 * inputs(148, 16)
+    yg = np.empty((16, 30), np.float32)
+    refi.lib.iris_group_norm(P(yg), P(np.ascontiguousarray(gimg.T)), P(gamma.astype(np.float32)), P(beta.astype(np.float32)),
+                             C.c_int(1), C.c_int(16), C.c_int(5), C.c_int(6), C.c_int(4), C.c_float(1e-6))
+    g["ops_group_norm"] = np.ascontiguousarray(yg.T)
+    uimg = inputs(149, 12, 5)
+    yu = np.empty((5, 6, 8), np.float32)
+    refi.lib.iris_upsample_nearest(P(yu), P(np.ascontiguousarray(uimg.T)), C.c_int(1), C.c_int(5), C.c_int(3), C.c_int(4), C.c_int(2), C.c_int(2))
+    g["ops_upsample2x"] = np.ascontiguousarray(yu.reshape(5, 48).T)
     out = os.path.join(HERE, "ref_vectors.npz")
     np.savez_compressed(out, **g)
     print("wrote", out, os.path.getsize(out), "bytes,", len(g), "arrays")

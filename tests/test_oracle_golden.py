@@ -7,6 +7,8 @@ import os
 import numpy as np
 import pytest
 
+import oracle as O
+
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_vectors.npz")
 
 
@@ -102,3 +104,19 @@ def test_qwen3_causal_gqa_chain(orc, gold):
     np.testing.assert_allclose(k, gold["qwen3_k"], rtol=1e-4, atol=1e-5)
     got = orc.attention_strided(q, k, v, heads, kv, 1 / np.sqrt(hd), causal=True, key_mask=mask)
     np.testing.assert_allclose(got, gold["qwen3_attention"], rtol=2e-4, atol=2e-5)
+
+
+def test_other_device_operators(orc, gold):
+    """The oracle's device-operator restatements against outputs of the reference's CPU twins
+    (written by make_golden.py; the reference works in NCHW, the fixtures are stored channels-last)."""
+    xl, Wl = O.f32_to_bf16(inputs(140, 7, 96)), O.f32_to_bf16(inputs(141, 33, 96) * 0.1)
+    np.testing.assert_allclose(orc.dev_linear(xl, Wl), gold["ops_linear"], atol=2e-5)
+    np.testing.assert_allclose(orc.dev_silu(inputs(142, 500) * 3), gold["ops_silu"], atol=1e-6)
+    h, w, cin, cout, k = 6, 5, 8, 4, 3
+    img = O.bf16_to_f32(O.f32_to_bf16(inputs(143, h * w, cin)))
+    wt = O.f32_to_bf16(inputs(144, cout, k * k * cin) * 0.2)
+    np.testing.assert_allclose(orc.dev_conv2d(img, wt, inputs(145, cout), h, w, k, 1, 1, 1), gold["ops_conv2d"], atol=2e-5)
+    gimg = inputs(146, 30, 16) * 2 + 0.5
+    gamma, beta = (1 + 0.1 * inputs(147, 16)).astype(np.float32), (0.1 * inputs(148, 16)).astype(np.float32)
+    np.testing.assert_allclose(orc.dev_group_norm(gimg, gamma, beta, 4, 1e-6, 0), gold["ops_group_norm"], atol=1e-5)
+    np.testing.assert_array_equal(orc.dev_upsample2x(inputs(149, 12, 5), 3, 4), gold["ops_upsample2x"])
