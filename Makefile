@@ -16,7 +16,7 @@ HIPFLAGS = -O3 --offload-arch=$(GPU_ARCH) -fPIC -std=c++17 -Xclang -target-featu
 CFLAGS   = -O2 -fPIC -Wall -Wextra -std=c11 -I$(CSRC) -Iinclude -I$(ROCM_HOME)/include
 
 HIP_SRCS = $(CSRC)/qknorm_rope.hip $(CSRC)/fa_fwd_gfx950.hip $(CSRC)/fa_fwd_sliced_gfx950.hip $(CSRC)/attn_generic.hip \
-           $(CSRC)/ew_norm_ops.hip $(CSRC)/gemm_conv_gfx950.hip
+           $(CSRC)/ew_norm_ops.hip $(CSRC)/gemm_conv_gfx950.hip $(CSRC)/rope_tables.hip
 HIP_OBJS = $(HIP_SRCS:.hip=.o)
 
 .PHONY: rocm oracle clean test-cpu test-gpu bench ctest
@@ -24,7 +24,7 @@ rocm: $(OUT) iris_c_amd/libiris_microbench.so
 
 # C-language parity program: host C over the ABI, checked against the oracle (run by the GPU tests)
 ctest: tests/c_abi_parity.bin
-tests/c_abi_parity.bin: tests/c_abi_parity.c include/iris_dev.h oracle/iris_oracle.h $(OUT) oracle/libiris_oracle.so
+tests/c_abi_parity.bin: tests/c_abi_parity.c include/iris_dev.h include/iris_rope.h oracle/iris_oracle.h $(OUT) oracle/libiris_oracle.so
 	$(CC) -O2 -Wall -Wextra -std=c11 -Iinclude -Ioracle -o $@ $< -Liris_c_amd -liris_dev -Loracle -liris_oracle \
 	    -Wl,-rpath,'$$ORIGIN/../iris_c_amd' -Wl,-rpath,'$$ORIGIN/../oracle' -Wl,-rpath,$(ROCM_HOME)/lib -lm
 
@@ -38,11 +38,16 @@ iris_c_amd/libiris_microbench.so: $(CSRC)/microbench.hip
 $(CSRC)/%.o: $(CSRC)/%.hip $(CSRC)/iris_kernels_hip.h
 	$(HIPCC) $(HIPFLAGS) -c $< -o $@
 
-$(CSRC)/iris_rocm.o: $(CSRC)/iris_rocm.c include/iris_dev.h $(CSRC)/iris_kernels_hip.h
+HOST_HDRS = include/iris_dev.h include/iris_rope.h $(CSRC)/iris_kernels_hip.h $(CSRC)/iris_rope_internal.h
+$(CSRC)/iris_rocm.o: $(CSRC)/iris_rocm.c $(HOST_HDRS)
 	$(CC) $(CFLAGS) -c $< -o $@
 
-$(OUT): $(HIP_OBJS) $(CSRC)/iris_rocm.o
-	$(HIPCC) --offload-arch=$(GPU_ARCH) -shared -o $@ $^ -L$(ROCM_HOME)/lib -lamdhip64
+# host builders of the rotary tables: IEEE arithmetic (no -ffast-math), their values are compared bit for bit
+$(CSRC)/iris_rope_tables.o: $(CSRC)/iris_rope_tables.c $(HOST_HDRS)
+	$(CC) $(CFLAGS) -c $< -o $@
+
+$(OUT): $(HIP_OBJS) $(CSRC)/iris_rocm.o $(CSRC)/iris_rope_tables.o
+	$(HIPCC) --offload-arch=$(GPU_ARCH) -shared -o $@ $^ -L$(ROCM_HOME)/lib -lamdhip64 -lm
 
 oracle:
 	$(MAKE) -C oracle all

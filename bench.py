@@ -13,7 +13,9 @@ Prints ONE JSON line. `value` is attention TFLOP/s over the whole step
 attention kernel alone, timed with HIP events on the library's stream.
 `norm_rope` reports the bandwidth-bound kernel the same way. `shapes` lists
 latency / TFLOP/s / GB/s for every benchmark configuration, `other_ops` the
-other device operators at this configuration's shapes. `cpu_baseline`
+other device operators at this configuration's shapes, `rope_tables` the
+time to build one forward pass's rotary tables (host builder + upload, and
+the device generator). `cpu_baseline`
 times the reference's BLAS-build CPU structure on this host's cores.
 """
 import argparse
@@ -44,49 +46,31 @@ def to_bf16(x):
     return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
-def rope_table(pos_axes, dims, theta):
-    """cos/sin [seq, sum(dims)/2] for integer positions per axis (closed form)."""
-    cs, sn = [], []
-    for p, d in zip(pos_axes, dims):
-        freq = (1.0 / np.power(np.float32(theta), np.arange(0, d, 2, dtype=np.float32) / np.float32(d))).astype(np.float32)
-        ang = p.astype(np.float32)[:, None] * freq[None, :]
-        cs.append(np.cos(ang)); sn.append(np.sin(ang))
-    return np.concatenate(cs, 1).astype(np.float32), np.concatenate(sn, 1).astype(np.float32)
-
-
-def flux2_positions(txt, grid, refs):
-    img = grid * grid
-    seq = txt + img * (1 + refs)
-    T, H, Wd, L = (np.zeros(seq, np.int32) for _ in range(4))
-    L[:txt] = np.arange(txt)
-    ys, xs = np.divmod(np.arange(img), grid)
-    for i in range(1 + refs):
-        sl = slice(txt + i * img, txt + (i + 1) * img)
-        H[sl], Wd[sl], T[sl] = ys, xs, 10 * i
-    return [T, H, Wd, L]
-
-
 def make_config(name, rng):
-    """Synthetic data of one benchmark configuration (numpy PCG64 normals)."""
+    """Synthetic data of one benchmark configuration (numpy PCG64 normals); rotary tables from the
+    library's own host builders (include/iris_rope.h)."""
+    from iris_c_amd.rope import RopeTables
+    rt = RopeTables()
     hd = 128
     c = dict(name=name, hd=hd, causal=False, key_mask=None, split_half=0, eps=1e-6)
     if name in ("C1", "C2", "C5"):
         txt, grid, refs, sigma = {"C1": (64, 16, 0, 1.0), "C2": (512, 64, 0, 1 / np.sqrt(128)), "C5": (512, 64, 2, 1.0)}[name]
         c.update(heads=24, kv_heads=24, seq=txt + grid * grid * (1 + refs), sigma=[sigma])
-        c["cos"], c["sin"] = rope_table(flux2_positions(txt, grid, refs), [32, 32, 32, 32], 2000.0)
+        c["layout"] = (txt, grid, grid, [(grid, grid)] * refs)
+        c["cos"], c["sin"] = rt.flux2_tables(*c["layout"])
     elif name in ("C3-cond", "C3-uncond"):
         seq = 4096 + 256
         c.update(heads=30, kv_heads=30, seq=seq, eps=1e-5, sigma=[1 / np.sqrt(128)] if name == "C3-cond" else [0.1])
-        pos = [np.r_[np.full(4096, 257), 1 + np.arange(256)], np.r_[np.arange(4096) // 64, np.zeros(256)],
-               np.r_[np.arange(4096) % 64, np.zeros(256)]]
-        c["cos"], c["sin"] = rope_table([p.astype(np.int32) for p in pos], [32, 48, 48], 256.0)
+        pos, _, ip, cp = rt.zimage_positions(img_seq=4096, wt=64, cap_seq=256)      # [image | caption]
+        assert ip + cp == seq
+        c["cos"], c["sin"] = rt.zimage_tables(pos, (32, 48, 48), (1536, 512, 512), 256.0)
         if name == "C3-uncond":
             length = int(rng.integers(16, 257))
             c["key_mask"] = np.r_[np.ones(4096), np.arange(256) < length].astype(np.int32)
     elif name == "C4":
         seq = 512
         c.update(heads=32, kv_heads=8, seq=seq, causal=True, split_half=1, sigma=[1.0])
-        c["cos"], c["sin"] = rope_table([np.arange(seq, dtype=np.int32)], [128], 1e6)
+        c["cos"], c["sin"] = rt.qwen3_tables(seq, 128, 1e6)
         c["key_mask"] = (np.arange(seq) < int(rng.integers(8, 513))).astype(np.int32)
     else:
         raise ValueError(name)
@@ -238,6 +222,34 @@ def other_ops(dev, hip, stream, rng):
     return res
 
 
+def rope_table_times(dev, c):
+    """Building the rotary tables of one forward pass of the bench configuration (wall clock, host side
+    included): the library's host builder + upload, and its device generator (positions staged, kernel run)."""
+    from iris_c_amd.rope import RopeTables
+    lib, rt = dev.lib, RopeTables(dev.lib)
+    txt, gh, gw, refs = c["layout"]
+    rows, nbytes = c["seq"], c["cos"].nbytes
+    dc, ds = lib.iris_dev_alloc(nbytes), lib.iris_dev_alloc(nbytes)
+
+    def best(fn, n=5):
+        ts = []
+        for _ in range(n):
+            t0 = time.perf_counter(); fn(); lib.iris_dev_sync(); ts.append(time.perf_counter() - t0)
+        return min(ts) * 1e3
+
+    def host():
+        cos, sin = rt.flux2_tables(txt, gh, gw, refs)
+        lib.iris_dev_upload(dc, cos.ctypes.data_as(_vp), nbytes)
+        lib.iris_dev_upload(ds, sin.ctypes.data_as(_vp), nbytes)
+
+    host_ms = best(host)
+    dev_ms = best(lambda: lib.iris_dev_rope_flux2_tables(dc, ds, txt, gh, gw, None, None, None, len(refs), 32, 2000.0))
+    dev.check()
+    lib.iris_dev_free(dc); lib.iris_dev_free(ds)
+    return {"rows": rows, "table_bytes": 2 * nbytes, "host_build_and_upload_ms": round(host_ms, 3),
+            "device_generate_ms": round(dev_ms, 3)}
+
+
 # ----------------------------------------------------------------------------- machine ceilings
 def microbench_lib():
     mb = C.CDLL(os.path.join(ROOT, "iris_c_amd", "libiris_microbench.so"))
@@ -326,12 +338,16 @@ def cpu_baseline(c):
     t1 = time.perf_counter()
     base.norm_rope(x, c["wq"], c["cos"], c["sin"], c["eps"], c["split_half"])
     dn = time.perf_counter() - t1
+    t2 = time.perf_counter()
+    oracle.oracle().flux2_joint_tables(*c["layout"])     # the reference's routine restated: libm on every entry
+    dtab = time.perf_counter() - t2
     return {"value": round(flops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "sample": f"{calls} full {c['name']} attention calls ({c['heads']}h x {c['seq']} tok, f32), mean of the last "
                       f"{calls - 1}: {dt:.2f} s each; "
                       f"sgemm from {os.path.basename(base.provider)}; host has {cores} CPUs online",
             "attention_seconds": round(dt, 3),
-            "norm_rope_gbps": round(2 * x.nbytes / dn / 1e9, 3), "norm_rope_cores": 1}
+            "norm_rope_gbps": round(2 * x.nbytes / dn / 1e9, 3), "norm_rope_cores": 1,
+            "rope_tables_ms": round(dtab * 1e3, 2)}
 
 
 # ----------------------------------------------------------------------------- main
@@ -433,6 +449,7 @@ def main():
 
     if not args.no_shapes:
         out["other_ops"] = other_ops(dev, hip, stream, rng)
+        out["rope_tables"] = rope_table_times(dev, c2)
     if not args.no_machine:
         out["machine"] = machine_ceilings(dev, hip, stream)
         # The ABI takes device pointers, so `value` has no host transfer in it. For a caller that had the

@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(HERE, "libiris_dev.so")
 _vp, _i, _f, _sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
 
 # name -> (restype, argtypes); the exported C ABI, one entry per declaration of include/iris_dev.h
+# and include/iris_rope.h
 ABI = {
     "iris_dev_init": (_i, []),
     "iris_dev_available": (_i, []),
@@ -48,6 +49,24 @@ ABI = {
     "iris_dev_stream": (_vp, []),
     "iris_dev_last_error": (_i, []),
     "iris_dev_last_kernel": (C.c_char_p, []),
+    # include/iris_rope.h: host builders (run without a GPU) ...
+    "iris_rope_expand_i32": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp, _f]),
+    "iris_rope_expand_f64": (_i, [_vp, _vp, _vp, _i, _i, _vp, _f]),
+    "iris_rope_joint_rows": (_i, [_i, _i, _i, _vp, _vp, _i]),
+    "iris_rope_flux2_positions": (None, [_vp, _i, _i, _i, _vp, _vp, _vp, _i]),
+    "iris_rope_flux2_tables": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _i, _i, _f]),
+    "iris_rope_flux3_positions": (None, [_vp, _i, _i, _i, _vp, _vp, _i]),
+    "iris_rope_flux3_tables": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _f]),
+    "iris_rope_zimage_positions": (None, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    "iris_rope_zimage_tables": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _f]),
+    "iris_rope_qwen3_tables": (_i, [_vp, _vp, _vp, _i, _i, _f, _i]),
+    # ... and the same tables generated on the device
+    "iris_dev_rope_expand_i32": (None, [_vp, _vp, _vp, _i, _i, _vp, _vp, _f]),
+    "iris_dev_rope_expand_f64": (None, [_vp, _vp, _vp, _i, _i, _vp, _f]),
+    "iris_dev_rope_flux2_tables": (None, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _i, _i, _f]),
+    "iris_dev_rope_flux3_tables": (None, [_vp, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _f]),
+    "iris_dev_rope_zimage_tables": (None, [_vp, _vp, _vp, _i, _vp, _vp, _f]),
+    "iris_dev_rope_qwen3_tables": (None, [_vp, _vp, _vp, _i, _i, _f, _i]),
 }
 
 

@@ -80,6 +80,13 @@ int iris_hip_conv2d(void *stream, uint16_t *scratch, size_t scratch_bytes, float
                     const uint16_t *w, const float *bias, int h, int width, int cin, int cout, int k,
                     int stride, int pad_before, int pad_after);
 
+/* Rotary tables [seq, half] from positions [seq, naxes] (int32, or float when use_double) and
+ * one frequency per column (float, or double when use_double); col_axis[half] names the axis of
+ * each column. All pointers are device memory; freq 8-byte aligned when use_double. */
+int iris_hip_rope_tables(void *stream, float *cos_t, float *sin_t, const void *freq,
+                         const int *col_axis, const void *pos, int seq, int half, int naxes,
+                         int use_double);
+
 #ifdef __cplusplus
 }
 #endif

@@ -20,6 +20,8 @@
 
 #include "iris_dev.h"
 #include "iris_kernels_hip.h"
+#include "iris_rope.h"
+#include "iris_rope_internal.h"
 
 static int g_ready = 0;
 static char g_name[640] = "none";
@@ -32,6 +34,9 @@ static const char *g_last_kernel = "none";
 static uint16_t *g_conv_scratch = NULL;
 static float *g_gn_scratch = NULL;
 static size_t g_gn_scratch_floats = 0;
+/* positions and column frequencies of the rotary tables being generated */
+static void *g_rope_stage = NULL;
+static size_t g_rope_stage_bytes = 0;
 
 static void fail(int code, const char *what, const char *detail) {
     g_last_error = code ? code : -1;
@@ -87,9 +92,12 @@ void iris_dev_cleanup(void) {
     check(hipStreamSynchronize(g_stream), "sync");
     if (g_conv_scratch) check(hipFree(g_conv_scratch), "free");
     if (g_gn_scratch) check(hipFree(g_gn_scratch), "free");
+    if (g_rope_stage) check(hipFree(g_rope_stage), "free");
     g_conv_scratch = NULL;
     g_gn_scratch = NULL;
     g_gn_scratch_floats = 0;
+    g_rope_stage = NULL;
+    g_rope_stage_bytes = 0;
     check(hipStreamDestroy(g_stream), "stream destroy");
     g_stream = NULL;
     g_ready = 0;
@@ -328,4 +336,109 @@ void iris_dev_group_norm(float *out, const float *in, const float *gamma, const 
 void iris_dev_upsample2x(float *out, const float *in, int h, int width, int c) {
     if (h <= 0 || width <= 0 || c <= 0) return;
     LAUNCH("upsample2x", iris_hip_upsample2x(g_stream, out, in, h, width, c));
+}
+
+/* ---- rotary tables generated on the device (include/iris_rope.h) ---- */
+
+/* Stages [freq: half x 8 B | col_axis: half x 4 B | pos: seq x naxes x 4 B] in one upload and
+ * launches the table kernel. pos is int32 (use_double 0) or float (use_double 1). */
+static void rope_tables(const char *what, float *d_cos, float *d_sin, const void *pos, int seq, int naxes,
+                        const int *axis_dims, const int *axis_lens, float theta, int use_double) {
+    if (!need_ready(what)) return;
+    if (!iris_rope_axes_ok_(seq, naxes, axis_dims) || (seq && (!d_cos || !d_sin || !pos))) {
+        fail(-1, what, "bad arguments");
+        return;
+    }
+    size_t half = 0;
+    for (int a = 0; a < naxes; a++) half += (size_t)(axis_dims[a] / 2);
+    if (!seq || !half) return;
+    const size_t freq_bytes = half * 8, axis_bytes = (half * 4 + 7) & ~(size_t)7;
+    const size_t pos_bytes = (size_t)seq * naxes * 4, total = freq_bytes + axis_bytes + pos_bytes;
+    unsigned char *blob = malloc(total);
+    if (!blob) { fail(-1, what, "out of host memory"); return; }
+    int *col_axis = (int *)(blob + freq_bytes);
+    size_t col = 0;
+    for (int a = 0; a < naxes; a++)
+        for (int j = 0; j < axis_dims[a] / 2; j++, col++) {
+            if (use_double) ((double *)blob)[col] = iris_rope_freq64_(theta, j, axis_dims[a]);
+            else ((float *)blob)[col] = iris_rope_freq32_(theta, j, axis_dims[a]);
+            col_axis[col] = a;
+        }
+    memcpy(blob + freq_bytes + axis_bytes, pos, pos_bytes);
+    if (axis_lens) {                       /* bounded axes: a position outside [0, len) does not rotate */
+        int *p = (int *)(blob + freq_bytes + axis_bytes);
+        for (size_t i = 0; i < (size_t)seq * naxes; i++)
+            if (p[i] < 0 || p[i] >= axis_lens[i % naxes]) p[i] = 0;
+    }
+    if (total > g_rope_stage_bytes) {
+        if (g_rope_stage) {
+            check(hipStreamSynchronize(g_stream), "sync");
+            check(hipFree(g_rope_stage), "free");
+        }
+        g_rope_stage = NULL;
+        g_rope_stage_bytes = 0;
+        if (hipMalloc(&g_rope_stage, total) != hipSuccess) {
+            (void)hipGetLastError();
+            g_rope_stage = NULL;
+            free(blob);
+            fail(-1, what, "out of device memory for the position staging buffer");
+            return;
+        }
+        g_rope_stage_bytes = total;
+    }
+    /* stream order keeps an earlier table kernel's reads ahead of this overwrite of the staging buffer */
+    int ok = check(hipMemcpyAsync(g_rope_stage, blob, total, hipMemcpyHostToDevice, g_stream), "upload") &&
+             check(hipStreamSynchronize(g_stream), "sync");
+    free(blob);
+    if (!ok) return;
+    const unsigned char *d = g_rope_stage;
+    int err = iris_hip_rope_tables(g_stream, d_cos, d_sin, d, (const int *)(d + freq_bytes),
+                                   d + freq_bytes + axis_bytes, seq, (int)half, naxes, use_double);
+    if (err) check((hipError_t)err, "rope tables launch");
+}
+
+void iris_dev_rope_expand_i32(float *d_cos, float *d_sin, const int *pos, int seq, int naxes,
+                              const int *axis_dims, const int *axis_lens, float theta) {
+    rope_tables("rope_expand_i32", d_cos, d_sin, pos, seq, naxes, axis_dims, axis_lens, theta, 0);
+}
+
+void iris_dev_rope_expand_f64(float *d_cos, float *d_sin, const float *pos, int seq, int naxes,
+                              const int *axis_dims, float theta) {
+    rope_tables("rope_expand_f64", d_cos, d_sin, pos, seq, naxes, axis_dims, NULL, theta, 1);
+}
+
+void iris_dev_rope_flux2_tables(float *d_cos, float *d_sin, int txt_seq, int img_h, int img_w,
+                                const int *ref_h, const int *ref_w, const int *ref_t, int num_refs,
+                                int axis_dim, float theta) {
+    const int rows = iris_rope_joint_rows(txt_seq, img_h, img_w, ref_h, ref_w, num_refs);
+    int *pos = rows < 0 ? NULL : malloc(sizeof(int) * 4 * (size_t)(rows ? rows : 1));
+    if (!pos) { fail(-1, "rope_flux2_tables", "bad sizes or out of host memory"); return; }
+    iris_rope_flux2_positions(pos, txt_seq, img_h, img_w, ref_h, ref_w, ref_t, num_refs);
+    const int dims[4] = { axis_dim, axis_dim, axis_dim, axis_dim };
+    rope_tables("rope_flux2_tables", d_cos, d_sin, pos, rows, 4, dims, NULL, theta, 0);
+    free(pos);
+}
+
+void iris_dev_rope_flux3_tables(float *d_cos, float *d_sin, int txt_seq, int img_h, int img_w,
+                                const int *ref_h, const int *ref_w, int num_refs,
+                                const int axes_dim[4], float theta) {
+    const int rows = iris_rope_joint_rows(txt_seq, img_h, img_w, ref_h, ref_w, num_refs);
+    float *pos = rows < 0 ? NULL : malloc(sizeof(float) * 4 * (size_t)(rows ? rows : 1));
+    if (!pos) { fail(-1, "rope_flux3_tables", "bad sizes or out of host memory"); return; }
+    iris_rope_flux3_positions(pos, txt_seq, img_h, img_w, ref_h, ref_w, num_refs);
+    rope_tables("rope_flux3_tables", d_cos, d_sin, pos, rows, 4, axes_dim, NULL, theta, 1);
+    free(pos);
+}
+
+void iris_dev_rope_zimage_tables(float *d_cos, float *d_sin, const int *pos3, int seq,
+                                 const int axes_dims[3], const int axes_lens[3], float theta) {
+    rope_tables("rope_zimage_tables", d_cos, d_sin, pos3, seq, 3, axes_dims, axes_lens, theta, 0);
+}
+
+void iris_dev_rope_qwen3_tables(float *d_cos, float *d_sin, const int *attention_mask, int seq,
+                                int head_dim, float theta, int pad_at_one) {
+    int *pos = seq < 0 ? NULL : iris_rope_qwen3_positions_(attention_mask, seq, pad_at_one);
+    if (!pos) { fail(-1, "rope_qwen3_tables", "bad sizes or out of host memory"); return; }
+    rope_tables("rope_qwen3_tables", d_cos, d_sin, pos, seq, 1, &head_dim, NULL, theta, 0);
+    free(pos);
 }

@@ -1,0 +1,16 @@
+/*
+ * Shared between the host table builders (iris_rope_tables.c) and the device
+ * entries (iris_rocm.c), so that both take their column frequencies and
+ * positions from the same code. Not part of the public interface.
+ */
+#ifndef IRIS_ROPE_INTERNAL_H
+#define IRIS_ROPE_INTERNAL_H
+
+float iris_rope_freq32_(float theta, int j, int dim);
+double iris_rope_freq64_(float theta, int j, int dim);
+/* malloc'd positions of the text encoder's rows, NULL on failure */
+int *iris_rope_qwen3_positions_(const int *attention_mask, int seq, int pad_at_one);
+/* argument check of the expansion routines: 1 = usable */
+int iris_rope_axes_ok_(int seq, int naxes, const int *axis_dims);
+
+#endif

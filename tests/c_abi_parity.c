@@ -5,7 +5,10 @@
  * (iris_transformer_flux.c:3834-3839): per-head RMSNorm + RoPE on Q, on K,
  * then joint attention, on the fused q|k|v row buffer, through the entry
  * points of include/iris_dev.h only, and compares every output element with
- * the CPU oracle run on the same inputs. A second pass covers the causal
+ * the CPU oracle run on the same inputs. The device side takes its rotary
+ * tables from the library's own generators (include/iris_rope.h), the oracle
+ * side from the oracle's, so the table builders are part of what is checked.
+ * A second pass covers the causal
  * grouped-KV + padding-mask form of the text encoder (iris_qwen3.c:1590-1596),
  * a third the single 512-wide head of the VAE (iris_vae.c:1112-1124).
  *
@@ -18,6 +21,7 @@
 #include <string.h>
 
 #include "iris_dev.h"
+#include "iris_rope.h"
 #include "iris_oracle.h"
 
 static int failures = 0;
@@ -52,9 +56,11 @@ static void *to_device(const void *src, size_t bytes) {
     return d;
 }
 
-/* norm+rope on Q and K, then attention; rows = [q | k | v], strides in elements */
+/* norm+rope on Q and K, then attention; rows = [q | k | v], strides in elements.
+ * d_cos / d_sin: device tables from the library; cos_t / sin_t: the oracle's tables for the same rows. */
 static void block_case(const char *name, int seq, int heads, int kv_heads, int split_half, int causal,
-                       const int *mask, const float *cos_t, const float *sin_t, float eps, uint64_t seed) {
+                       const int *mask, float *d_cos, float *d_sin, const float *cos_t, const float *sin_t,
+                       float eps, uint64_t seed) {
     const int hd = 128, qd = heads * hd, kd = kv_heads * hd, ldi = qd + 2 * kd, ldo = qd;
     orc_rng_t g;
     orc_rng_seed(&g, seed);
@@ -68,7 +74,6 @@ static void block_case(const char *name, int seq, int heads, int kv_heads, int s
     /* device */
     uint16_t *d_rows = to_device(rows, (size_t)seq * ldi * 2);
     float *d_wq = to_device(wq, sizeof wq), *d_wk = to_device(wk, sizeof wk);
-    float *d_cos = to_device(cos_t, (size_t)seq * 64 * 4), *d_sin = to_device(sin_t, (size_t)seq * 64 * 4);
     int *d_mask = mask ? to_device(mask, (size_t)seq * sizeof(int)) : NULL;
     uint16_t *d_out = iris_dev_alloc((size_t)seq * ldo * 2);
     iris_dev_head_norm_rope(d_rows, ldi, d_wq, d_cos, d_sin, seq, heads, hd, eps, split_half);
@@ -132,8 +137,17 @@ int main(void) {
         const int txt = 40, gh = 12, gw = 12, seq = txt + gh * gw;
         float *c = malloc((size_t)seq * 64 * 4), *s = malloc((size_t)seq * 64 * 4);
         orc_flux2_joint_tables(c, s, txt, gh, gw, NULL, NULL, 0, 32, 2000.0f);
-        block_case("joint 24h", seq, 24, 24, 0, 0, NULL, c, s, 1e-6f, 20250101);
-        free(c); free(s);
+        float *hc = malloc((size_t)seq * 64 * 4), *hs = malloc((size_t)seq * 64 * 4);
+        if (iris_rope_joint_rows(txt, gh, gw, NULL, NULL, 0) != seq ||
+            iris_rope_flux2_tables(hc, hs, txt, gh, gw, NULL, NULL, NULL, 0, 32, 2000.0f) != 0 ||
+            memcmp(hc, c, (size_t)seq * 64 * 4) || memcmp(hs, s, (size_t)seq * 64 * 4)) {
+            printf("host flux2 tables differ from the oracle's\n");
+            failures++;
+        }
+        float *d_cos = iris_dev_alloc((size_t)seq * 64 * 4), *d_sin = iris_dev_alloc((size_t)seq * 64 * 4);
+        iris_dev_rope_flux2_tables(d_cos, d_sin, txt, gh, gw, NULL, NULL, NULL, 0, 32, 2000.0f);
+        block_case("joint 24h", seq, 24, 24, 0, 0, NULL, d_cos, d_sin, c, s, 1e-6f, 20250101);
+        free(c); free(s); free(hc); free(hs);
     }
     /* text encoder layer: causal, 32 query heads on 8 kv heads, split-half rotation, right padding */
     {
@@ -142,7 +156,9 @@ int main(void) {
         int *mask = malloc(seq * sizeof(int));
         for (int i = 0; i < seq; i++) mask[i] = i < len;
         orc_qwen3_rope_table(c, s, mask, seq, 128, 1e6f, 0);
-        block_case("causal gqa 32/8", seq, 32, 8, 1, 1, mask, c, s, 1e-6f, 20250104);
+        float *d_cos = iris_dev_alloc((size_t)seq * 64 * 4), *d_sin = iris_dev_alloc((size_t)seq * 64 * 4);
+        iris_dev_rope_qwen3_tables(d_cos, d_sin, mask, seq, 128, 1e6f, 0);
+        block_case("causal gqa 32/8", seq, 32, 8, 1, 1, mask, d_cos, d_sin, c, s, 1e-6f, 20250104);
         free(c); free(s); free(mask);
     }
     vae_case(300, 20250107);

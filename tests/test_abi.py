@@ -18,9 +18,12 @@ def lib():
 
 
 def declared_functions():
-    text = open(os.path.join(ROOT, "include", "iris_dev.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return re.findall(r"\b(iris_dev_\w+)\s*\(", text)
+    names = []
+    for header in ("iris_dev.h", "iris_rope.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names += re.findall(r"\b(iris_(?:dev|rope)_\w+)\s*\(", text)
+    return names
 
 
 def test_every_declared_symbol_is_exported_and_bound(lib):
@@ -53,6 +56,9 @@ def test_no_gpu_means_no_silent_fallback(lib):
     lib.iris_dev_attention(None, 0, None, None, None, 0, 4, 4, 1, 1, 128, 1.0, 0, None)
     assert lib.iris_dev_last_error() != 0
     lib.iris_dev_head_norm_rope(None, 0, None, None, None, 4, 1, 128, 1e-6, 0)
+    assert lib.iris_dev_last_error() != 0
+    # device-side table generation likewise; the host builders of the same header need no device
+    lib.iris_dev_rope_qwen3_tables(None, None, None, 4, 128, 1e6, 0)
     assert lib.iris_dev_last_error() != 0
 
 
