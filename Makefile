@@ -6,6 +6,7 @@
 ROCM_HOME ?= /opt/rocm
 HIPCC     ?= $(ROCM_HOME)/bin/hipcc
 CC        ?= gcc
+CXX       ?= g++
 GPU_ARCH  ?= gfx950
 
 CSRC   = iris_c_amd/csrc
@@ -46,8 +47,12 @@ $(CSRC)/iris_rocm.o: $(CSRC)/iris_rocm.c $(HOST_HDRS)
 $(CSRC)/iris_rope_tables.o: $(CSRC)/iris_rope_tables.c $(HOST_HDRS)
 	$(CC) $(CFLAGS) -c $< -o $@
 
-$(OUT): $(HIP_OBJS) $(CSRC)/iris_rocm.o $(CSRC)/iris_rope_tables.o
-	$(HIPCC) --offload-arch=$(GPU_ARCH) -shared -o $@ $^ -L$(ROCM_HOME)/lib -lamdhip64 -lm
+# glue to the vendor GEMM library: host C++ only; the library itself is opened with dlopen at run time
+$(CSRC)/linear_hipblaslt.o: $(CSRC)/linear_hipblaslt.cpp $(CSRC)/iris_kernels_hip.h
+	$(CXX) -O2 -fPIC -Wall -Wextra -std=c++17 -I$(CSRC) -I$(ROCM_HOME)/include -c $< -o $@
+
+$(OUT): $(HIP_OBJS) $(CSRC)/iris_rocm.o $(CSRC)/iris_rope_tables.o $(CSRC)/linear_hipblaslt.o
+	$(HIPCC) --offload-arch=$(GPU_ARCH) -shared -o $@ $^ -L$(ROCM_HOME)/lib -lamdhip64 -lm -ldl
 
 oracle:
 	$(MAKE) -C oracle all

@@ -200,9 +200,12 @@ def other_ops(dev, hip, stream, rng):
     y = lib.iris_dev_alloc(rows * 27648 * 4)
     for k, n in ((3072, 9216), (3072, 3072), (3072, 18432), (9216, 3072), (3072, 27648), (12288, 3072)):
         for name, fn in (("linear_f32", lib.iris_dev_linear_f32), ("linear_bf16", lib.iris_dev_linear_bf16)):
-            ms = timed(lambda i: fn(y, x, W, rows, k, n), 5)
-            res.append({"op": name, "shape": f"{rows}x{k}->{n}", "us": round(ms * 1e3, 1),
-                        "tflops": round(2 * rows * k * n / ms / 1e9, 1)})
+            for backend in (0, 1):            # 0: vendor GEMM library when present (the default), 1: own MFMA kernel
+                lib.iris_dev_linear_backend(backend)
+                ms = timed(lambda i: fn(y, x, W, rows, k, n), 5)
+                res.append({"op": name, "kernel": dev.last_kernel(), "shape": f"{rows}x{k}->{n}", "us": round(ms * 1e3, 1),
+                            "tflops": round(2 * rows * k * n / ms / 1e9, 1)})
+    lib.iris_dev_linear_backend(0)
     xf, af = _vp(y), _vp(y + rows * dim * 4)
     w1 = dev.to_device(np.ones(dim, np.float32))
     ob = _vp(x)

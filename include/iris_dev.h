@@ -147,6 +147,12 @@ int iris_dev_last_error(void);
  * call used: a static string such as "fa_hd128" or "generic". */
 const char *iris_dev_last_kernel(void);
 
+/* Which GEMM runs the linear layers. 0 (default): the vendor library hipBLASLt when it can be
+ * opened at run time and takes the problem, this library's own MFMA kernel otherwise
+ * (the reference's backend calls cuBLAS / hipBLAS for them, iris_cuda.cu:456-505);
+ * 1: always the own kernel. No counterpart in the reference. */
+void iris_dev_linear_backend(int which);
+
 #ifdef __cplusplus
 }
 #endif

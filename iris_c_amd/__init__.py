@@ -49,6 +49,7 @@ ABI = {
     "iris_dev_stream": (_vp, []),
     "iris_dev_last_error": (_i, []),
     "iris_dev_last_kernel": (C.c_char_p, []),
+    "iris_dev_linear_backend": (None, [_i]),
     # include/iris_rope.h: host builders (run without a GPU) ...
     "iris_rope_expand_i32": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp, _f]),
     "iris_rope_expand_f64": (_i, [_vp, _vp, _vp, _i, _i, _vp, _f]),

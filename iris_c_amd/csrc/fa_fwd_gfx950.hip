@@ -7,8 +7,13 @@
  *     out[i] = softmax_j(scale * q_i . k_j) v_j   over the valid keys j
  * where key j is valid when j < seq_k, (causal ? j <= i : true) and
  * (key_mask ? key_mask[j] != 0 : true). A query without valid keys gives a
- * zero row. P is rounded to bf16 for the P.V product while the row sum uses
- * the unrounded f32 values (reference iris_cuda.cu:656-665).
+ * zero row. P is rounded to bf16 for the P.V product (reference
+ * iris_cuda.cu:656-665). The row sum is taken over the same rounded values,
+ * on the matrix cores: one more product per tile with an all-ones A operand
+ * (+6 % MFMAs) replaces 32 additions per lane and the final cross-lane sum,
+ * and the weights of the output rows then add up to exactly one. The
+ * reference sums the unrounded f32 values; the two differ by the mean of the
+ * bf16 rounding errors of a row, far below one bf16 step of the output.
  *
  * Shape of the computation on CDNA4
  * ---------------------------------
@@ -112,7 +117,7 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
     return d;
 }
 
-/* Max (or sum) over the four lanes l%16, l%16+16, +32, +48 (one per 16-lane row); every one
+/* Max over the four lanes l%16, l%16+16, +32, +48 (one per 16-lane row); every one
  * of them gets the result. v_permlane16_swap(x, x) returns rows {0,0,2,2} and {1,1,3,3} of x,
  * v_permlane32_swap(x, x) rows {0,1,0,1} and {2,3,2,3}. */
 __device__ __forceinline__ float quad_group_max(float v) {
@@ -121,13 +126,6 @@ __device__ __forceinline__ float quad_group_max(float v) {
     auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false);
     return max3(__uint_as_float(b[0]), __uint_as_float(b[1]), __uint_as_float(b[1]));
 }
-__device__ __forceinline__ float quad_group_sum(float v) {
-    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    const float t = __uint_as_float(a[0]) + __uint_as_float(a[1]);
-    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false);
-    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
-}
-
 /* HBM -> registers: 16 B pieces of the 64-key tile whose first row is at
  * `kt` / `vt` (wave-uniform pointers), at this thread's four row offsets. */
 template <int NP>
@@ -211,7 +209,11 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     for (int db = 0; db < 8; db++)
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) o[db][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.0f, 0.0f};
+    float m_run[2] = {-INFINITY, -INFINITY};
+    /* row sums on the matrix cores: an all-ones A operand makes every row of the product the
+     * column sum of P^T, i.e. the sum of the lane's query over the tile's keys */
+    f32x4 l_acc[2] = {f32x4{0.0f, 0.0f, 0.0f, 0.0f}, f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
+    const bf16x8 ones = __builtin_bit_cast(bf16x8, u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
 
     int k_end = seq_k;
     if (CAUSAL) k_end = min(seq_k, q0 + BM);       /* keys beyond the last query of the block are never valid */
@@ -338,7 +340,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                 const float m_new = fmaxf(m_run[nb], mx[nb]);
                 const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - (m_new == -INFINITY ? 0.0f : m_new));
                 m_run[nb] = m_new;
-                l_run[nb] *= alpha;
+                l_acc[nb] *= alpha;
 #pragma unroll
                 for (int db = 0; db < 8; db++) o[db][nb] *= alpha;
             }
@@ -350,7 +352,6 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) {
             const float neg_m = m_run[nb] == -INFINITY ? 0.0f : -m_run[nb];   /* finite while every key so far is masked */
-            float psum = 0.0f;
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
                 float p[8];
@@ -360,9 +361,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                     p[4 + r] = __builtin_amdgcn_exp2f(fmaf(s[2 * ks + 1][nb][r], scale_log2, neg_m));
                 }
                 pw[ks][nb] = u32x4{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
-                psum += ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
             }
-            l_run[nb] += psum;                      /* per lane-group partial; the four are added at the end */
         }
 
         /* ---- O^T += V^T P^T : 2 k-steps of 32 keys x 8 dim blocks x 2 query blocks; the V^T
@@ -379,6 +378,8 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(1);
             const bf16x8 pb0 = __builtin_bit_cast(bf16x8, pw[ks][0]), pb1 = __builtin_bit_cast(bf16x8, pw[ks][1]);
+            l_acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb0, l_acc[0], 0, 0, 0);
+            l_acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb1, l_acc[1], 0, 0, 0);
 #pragma unroll
             for (int db = 0; db < 8; db++) {
                 s16x8 both = __builtin_shufflevector(lo[db], hi[db], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -393,7 +394,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     /* ---- normalise and store: the lane holds dims 16db + 4lg + {0..3} of its two queries ---- */
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
-        const float l_tot = quad_group_sum(l_run[nb]);
+        const float l_tot = l_acc[nb][0];              /* every row of the ones product is the full sum */
         const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
         const int qrow = qrow0 + 16 * nb;
         if (qrow < seq_q) {

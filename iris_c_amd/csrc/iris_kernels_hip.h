@@ -80,6 +80,14 @@ int iris_hip_conv2d(void *stream, uint16_t *scratch, size_t scratch_bytes, float
                     const uint16_t *w, const float *bias, int h, int width, int cin, int cout, int k,
                     int stride, int pad_before, int pad_after);
 
+/* Linear layer through hipBLASLt (linear_hipblaslt.cpp; the library is opened with dlopen at the
+ * first call). Returns 0 when the product was enqueued, 1 when the caller must use its own
+ * kernel: library absent, or no algorithm for this problem. Operands contiguous as above. */
+int iris_lt_linear(void *stream, void *y, int out_bf16, const uint16_t *x, const uint16_t *W,
+                   int rows, int in, int out);
+int iris_lt_available(void);
+void iris_lt_release(void);
+
 /* Rotary tables [seq, half] from positions [seq, naxes] (int32, or float when use_double) and
  * one frequency per column (float, or double when use_double); col_axis[half] names the axis of
  * each column. All pointers are device memory; freq 8-byte aligned when use_double. */

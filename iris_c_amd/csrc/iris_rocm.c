@@ -93,6 +93,7 @@ void iris_dev_cleanup(void) {
     if (g_conv_scratch) check(hipFree(g_conv_scratch), "free");
     if (g_gn_scratch) check(hipFree(g_gn_scratch), "free");
     if (g_rope_stage) check(hipFree(g_rope_stage), "free");
+    iris_lt_release();
     g_conv_scratch = NULL;
     g_gn_scratch = NULL;
     g_gn_scratch_floats = 0;
@@ -233,15 +234,35 @@ void iris_dev_f32_to_bf16(uint16_t *dst, const float *src, size_t n) {
     LAUNCH("f32_to_bf16", iris_hip_f32_to_bf16(g_stream, dst, src, n));
 }
 
+/* Plain GEMMs go to the vendor library when it is there and takes the problem (aligned operands,
+ * in % 8 == 0), to this library's own MFMA kernel otherwise. iris_dev_linear_backend(1) pins the
+ * own kernel. */
+static int g_linear_backend = 0;
+
+void iris_dev_linear_backend(int which) { g_linear_backend = which == 1 ? 1 : 0; }
+
+static int linear_by_library(void *y, int out_bf16, const uint16_t *x, const uint16_t *W, int rows, int in, int out) {
+    if (g_linear_backend != 0 || in % 8 != 0 || !aligned(y, 16) || !aligned(x, 16) || !aligned(W, 16)) return 0;
+    if (iris_lt_linear(g_stream, y, out_bf16, x, W, rows, in, out) != 0) return 0;
+    g_last_kernel = "linear_hipblaslt";
+    return 1;
+}
+
 void iris_dev_linear_f32(float *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out) {
     if (rows <= 0 || out <= 0) return;
     if (in <= 0) { fail(-1, "linear", "in must be positive"); return; }
+    if (!need_ready("linear")) return;
+    if (linear_by_library(y, 0, x, W, rows, in, out)) return;
+    g_last_kernel = "linear_mfma";
     LAUNCH("linear", iris_hip_linear_f32(g_stream, y, x, W, rows, in, out));
 }
 
 void iris_dev_linear_bf16(uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out) {
     if (rows <= 0 || out <= 0) return;
     if (in <= 0) { fail(-1, "linear", "in must be positive"); return; }
+    if (!need_ready("linear")) return;
+    if (linear_by_library(y, 1, x, W, rows, in, out)) return;
+    g_last_kernel = "linear_mfma";
     LAUNCH("linear", iris_hip_linear_bf16(g_stream, y, x, W, rows, in, out));
 }
 

@@ -44,13 +44,21 @@ def run(dev, fn, outs):
 # ------------------------------------------------------------------ linear
 @pytest.mark.parametrize("rows,k,out", [(1, 8, 1), (5, 64, 7), (128, 128, 128), (130, 200, 260), (333, 3072, 520), (64, 96, 64)])
 @pytest.mark.parametrize("out_bf16", [False, True])
-def test_linear(dev, orc, rows, k, out, out_bf16):
+@pytest.mark.parametrize("backend", ["library", "own"])
+def test_linear(dev, orc, rows, k, out, out_bf16, backend):
+    """Both GEMM paths: the vendor library (taken when present) and this library's own MFMA kernel."""
     x, W = O.f32_to_bf16(rnd((rows, k), rows + k)), O.f32_to_bf16(rnd((out, k), out, 0.05))
     want = orc.dev_linear(x, W)
     dx, dW = dev.put(x), dev.put(W)
     dy = dev.alloc(rows * out * (2 if out_bf16 else 4))
     fn = dev.lib.iris_dev_linear_bf16 if out_bf16 else dev.lib.iris_dev_linear_f32
-    got = run(dev, lambda: fn(dy, dx, dW, rows, k, out), [(dy, (rows, out), np.uint16 if out_bf16 else np.float32)])
+    dev.lib.iris_dev_linear_backend(1 if backend == "own" else 0)
+    try:
+        got = run(dev, lambda: fn(dy, dx, dW, rows, k, out), [(dy, (rows, out), np.uint16 if out_bf16 else np.float32)])
+        kernel = dev.dev.last_kernel()
+    finally:
+        dev.lib.iris_dev_linear_backend(0)
+    assert kernel == "linear_mfma" if backend == "own" else kernel in ("linear_hipblaslt", "linear_mfma")
     scale = np.sqrt(k) * 0.05
     if out_bf16:
         # round to nearest: half a bf16 ulp of the value, plus the f32 accumulation noise
@@ -67,10 +75,28 @@ def test_linear_unaligned_k_uses_the_scalar_kernel(dev, orc):
     np.testing.assert_allclose(got, orc.dev_linear(x, W), atol=1e-4)
 
 
-def test_linear_full_size_properties(dev, orc):
+def test_library_gemm_is_used_when_present(dev):
+    """On a ROCm machine hipBLASLt is there: an aligned linear layer must run through it (the own
+    kernel is the fallback, not the default), and pinning the own kernel must be honoured."""
+    rows, k, out = 64, 128, 64
+    dx, dW, dy = dev.put(np.zeros((rows, k), np.uint16)), dev.put(np.zeros((out, k), np.uint16)), dev.alloc(rows * out * 4)
+    dev.lib.iris_dev_linear_f32(dy, dx, dW, rows, k, out)
+    dev.check()
+    assert dev.dev.last_kernel() == "linear_hipblaslt"
+    dev.lib.iris_dev_linear_backend(1)
+    dev.lib.iris_dev_linear_f32(dy, dx, dW, rows, k, out)
+    dev.lib.iris_dev_linear_backend(0)
+    dev.check()
+    assert dev.dev.last_kernel() == "linear_mfma"
+    dev.free_all()
+
+
+@pytest.mark.parametrize("backend", ["library", "own"])
+def test_linear_full_size_properties(dev, orc, backend):
     """The QKV projection of the bench configuration (4608 x 3072 -> 9216): sampled entries against
     the oracle, and linearity in x: (x1 + x2) W == x1 W + x2 W for bf16-exact sums."""
     rows, k, out = 4608, 3072, 9216
+    dev.lib.iris_dev_linear_backend(1 if backend == "own" else 0)
     rng = np.random.default_rng(5)
     x = O.f32_to_bf16(rng.integers(-4, 5, (rows, k)).astype(np.float32) / 8)     # small dyadic values: exact in bf16
     W = O.f32_to_bf16(rng.integers(-4, 5, (out, k)).astype(np.float32) / 8)
@@ -79,6 +105,7 @@ def test_linear_full_size_properties(dev, orc):
     r = rng.integers(0, rows, 24); c = rng.integers(0, out, 24)
     xs, Ws = O.bf16_to_f32(x[r]).astype(np.float64), O.bf16_to_f32(W[c]).astype(np.float64)
     want = np.einsum("ik,ik->i", xs, Ws)
+    dev.lib.iris_dev_linear_backend(0)
     np.testing.assert_allclose(got[r, c], want, atol=1e-3)           # dyadic products: sums are exact in f32
     assert np.all(got == np.round(got * 64) / 64)                     # every entry is a multiple of 1/64
 
