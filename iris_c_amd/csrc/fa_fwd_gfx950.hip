@@ -17,13 +17,18 @@
  *
  * Shape of the computation on CDNA4
  * ---------------------------------
- * One workgroup = 8 waves = 256 queries of one head (4 waves = 128 queries
- * when that would leave CUs without work); each wave owns 32 queries for the
- * whole kernel, two waves share a SIMD. Keys/values stream through two LDS
- * stages in tiles of 64: while tile i is multiplied, tile i+1 moves
- * registers -> LDS and tile i+2 moves HBM -> registers; one barrier per tile.
- * Every wave reads the whole K and V tile, so 256 queries per workgroup mean
- * half the L2 -> LDS traffic and half the LDS writes per query of 128.
+ * One workgroup = WAVES (8, 4, 2 or 1) waves of 32 queries of one head; each
+ * wave owns its 32 queries for the whole kernel. 8 waves = 256 queries is the
+ * throughput shape (two waves share a SIMD, one workgroup per CU); the smaller
+ * ones are taken when the problem has too few queries to give every CU a
+ * large workgroup: a workgroup walks its key tiles one after the other, so a
+ * short sequence is bound by that latency and wants many small workgroups.
+ * Keys/values stream through LDS in tiles of 64 keys, 3 stages (2 below 8
+ * waves), and they go there directly: global_load_lds_dwordx4 copies
+ * HBM/L2 -> LDS without passing through registers, two tiles ahead of the
+ * one in use; one barrier per tile. Every wave reads the whole K and V tile,
+ * so 256 queries per workgroup mean half the L2 -> LDS traffic per query of
+ * 128.
  *
  * Both products are issued transposed so that a query is a COLUMN of every
  * accumulator: S^T = K Q^T (A = K tile from LDS, B = Q^T held in registers)
@@ -41,20 +46,24 @@
  * against 1.3 with 32x32x16 (a quarter of the accumulator registers read
  * and written per flop).
  *
- * LDS layout: K and V tiles row-major [64][128+16] bf16, 288 B rows.
- * ds_read_b128 serves 16 lanes per pass, and a pass is not 16 consecutive
- * lanes: with lanes 0-3, 12-15, 20-23, 24-27 in one pass (and the other
- * passes alike) the 16 lanes must fall in distinct 16 B bank windows. The
- * A operand read has lane l at row l%16, 16 B chunk l/16 (+ constants), so
- * the window is (row * 288/16 + chunk) % 16 = (2 row + chunk) % 16, which is
- * a bijection on every such pass; 272 B rows (row + chunk) gave a two-way
- * conflict on every read. The V^T operand comes from the LDS transpose read
+ * LDS layout: K and V tiles row-major [64][128] bf16, 256 B rows, unpadded
+ * (a direct load writes 64 lanes x 16 B to consecutive addresses, so rows
+ * cannot be padded); instead the 16 B chunk c of row r is kept in slot
+ * c ^ 2(r mod 8) of its row, the permutation being applied to the SOURCE
+ * address of the lane that fills the slot. ds_read_b128 serves 16 lanes per
+ * pass, and a pass is not 16 consecutive lanes: lanes 0-3, 12-15, 20-23,
+ * 24-27 go together (and the other passes alike), i.e. 16 different rows
+ * l%16 with chunk c0 + (0 or 1). Their slots (c0 + e) ^ 2(row mod 8) are 16
+ * distinct 16 B bank windows: rows that swizzle alike (r, r+8) sit in
+ * different halves of the pass and differ in e, all others differ in the
+ * swizzle. The V^T operand comes from the LDS transpose read
  * ds_read_b64_tr_b16, which hands lane i of a 16-lane group column i of a
  * 4-row x 16-column block: four consecutive keys of one head dim, exactly
  * the keys that four consecutive P^T registers of that lane belong to; it
- * serves 32 consecutive lanes (8 rows x 32 B) per pass, conflict-free when
- * the row stride is 32 B mod 256 B. Both hardware counters read zero bank
- * conflicts with this layout.
+ * serves 32 consecutive lanes (8 rows x 32 B) per pass, and the swizzle
+ * sends the eight rows to the eight different 32 B windows (it is even, so
+ * the two chunks of a 32 B piece stay adjacent). Hardware counters read zero
+ * bank conflicts for both.
  *
  * The running max is only raised when some query of the wave exceeds it by
  * more than 2^8 (the accumulators are then rescaled); otherwise the
@@ -82,22 +91,15 @@ namespace {
 /* A workgroup is WAVES (4 or 8) waves of 32 queries: BM = 32 * WAVES queries, 64 * WAVES threads. */
 constexpr int BN = 64;             /* keys per tile */
 constexpr int HD = 128;
-constexpr int KS = HD + 16;         /* K tile row stride in elements (288 B) */
-constexpr int VS = HD + 16;         /* V tile row stride in elements (288 B) */
+constexpr int KS = HD;              /* K and V tile rows are 256 B, unpadded: chunks are swizzled instead */
+constexpr int VS = HD;
 constexpr int K_TILE = BN * KS;    /* elements */
 constexpr int V_TILE = BN * VS;
-constexpr int STAGE = K_TILE + V_TILE;
+constexpr int STAGE = K_TILE + V_TILE;      /* 32 KB */
 constexpr int XCDS = 8;
 constexpr float RESCALE_THRESHOLD = 8.0f;   /* log2 units */
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-
-/* This thread's share of one K/V tile: NP = 1024 / threads pieces of 16 B of K and of V,
- * RSTEP = threads / 16 rows apart. */
-template <int NP>
-struct TileRegs {
-    u32x4 k[NP], v[NP];
-};
 
 /* Workgroup barrier that only waits for this wave's LDS traffic. __syncthreads()
  * would also wait for outstanding global loads (vmcnt(0)), i.e. for the tile
@@ -126,44 +128,61 @@ __device__ __forceinline__ float quad_group_max(float v) {
     auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false);
     return max3(__uint_as_float(b[0]), __uint_as_float(b[1]), __uint_as_float(b[1]));
 }
-/* HBM -> registers: 16 B pieces of the 64-key tile whose first row is at
- * `kt` / `vt` (wave-uniform pointers), at this thread's four row offsets. */
-template <int NP>
-__device__ __forceinline__ void fetch_tile(TileRegs<NP> &t, const uint16_t *kt, const uint16_t *vt,
-                                           const uint32_t *off) {
-    const char *kc = reinterpret_cast<const char *>(kt), *vc = reinterpret_cast<const char *>(vt);
+/* 16 B chunk c of tile row r lives in slot c ^ swz(r) of that row. */
+__device__ __forceinline__ int swz(int row) { return 2 * (row & 7); }
+
+/* HBM/L2 -> LDS without passing through registers: one global_load_lds_dwordx4 moves
+ * 64 lanes x 16 B into 1 KB of consecutive LDS (lane l at +16 l), i.e. four tile rows.
+ * A tile (K then V, 32 KB) is 32 such pieces, NI = 32 / WAVES per wave; piece g covers
+ * rows 4 (g % 16) .. +3 of K (g < 16) or V. The lane that fills slot s of row r fetches
+ * chunk s ^ swz(r) of that row: the swizzle is applied on the source side. Rows r and
+ * r + 8 swizzle alike, so a lane needs two source offsets in all: lane_off[g % 2], from
+ * the first row of the piece.
+ *
+ * Written as asm, not as __builtin_amdgcn_global_load_lds: the compiler cannot tell which
+ * stage a later LDS read touches and would wait for ALL outstanding requests (vmcnt(0))
+ * before every operand read, which serialises the pipeline. The waits are placed by hand
+ * (wait_vmcnt) where a tile is first needed. M0 carries the LDS address; nothing else in
+ * this kernel uses M0. */
+__device__ __forceinline__ uint32_t lds_address(const uint16_t *p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+
+template <int NI>
+__device__ __forceinline__ void load_tile(uint16_t *stage, const uint16_t *kt, const uint16_t *vt, int ldi,
+                                          const uint32_t (&lane_off)[2], int wave) {
 #pragma unroll
-    for (int c = 0; c < NP; c++) {
-        t.k[c] = *reinterpret_cast<const u32x4 *>(kc + off[c]);
-        t.v[c] = *reinterpret_cast<const u32x4 *>(vc + off[c]);
+    for (int j = 0; j < NI; j++) {
+        const int g = wave * NI + j;                       /* wave-uniform */
+        const uint16_t *src = (g < 16 ? kt : vt) + (size_t)(4 * (g & 15)) * ldi;      /* first row of the piece */
+        const uint16_t *dst = stage + (g < 16 ? 0 : K_TILE) + 4 * (g & 15) * KS;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     ::"s"(lds_address(dst)), "v"(lane_off[g & 1]), "s"(src) : "memory");
     }
 }
 
-/* Registers -> LDS stage. */
-template <int NP>
-__device__ __forceinline__ void store_tile(const TileRegs<NP> &t, uint16_t *stage, int tid) {
-    constexpr int RSTEP = 64 / NP;
-    const int row = tid >> 4, col = (tid & 15) * 8;
-    uint16_t *kp = &stage[row * KS + col], *vp = &stage[K_TILE + row * VS + col];
+/* The same for the last tile of a sequence whose rows run out before the tile does: rows
+ * past `last_row` (relative to the tile) are redirected to it. Their scores are masked and
+ * their probabilities are exactly zero, so the values never matter; they only must be
+ * finite, which any real row is. */
+template <int NI>
+__device__ __forceinline__ void load_tile_clamped(uint16_t *stage, const uint16_t *kt, const uint16_t *vt, int ldi,
+                                                  int last_row, int lane, int wave) {
 #pragma unroll
-    for (int c = 0; c < NP; c++) {
-        *reinterpret_cast<u32x4 *>(kp + c * RSTEP * KS) = t.k[c];
-        *reinterpret_cast<u32x4 *>(vp + c * RSTEP * VS) = t.v[c];
+    for (int j = 0; j < NI; j++) {
+        const int g = wave * NI + j;
+        const int row = 4 * (g & 15) + (lane >> 4);
+        const int chunk = (lane & 15) ^ swz(row);
+        const uint16_t *src = (g < 16 ? kt : vt) + (size_t)min(row, last_row) * ldi + 8 * chunk;
+        const uint16_t *dst = stage + (g < 16 ? 0 : K_TILE) + 4 * (g & 15) * KS;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                     ::"s"(lds_address(dst)), "v"(src) : "memory");
     }
 }
 
-/* Byte offsets of this thread's four rows of a tile starting at key k0; rows
- * past the end are redirected to the last valid row (their scores are masked
- * and their probabilities are exactly zero, so the values never matter). */
-template <int NP>
-__device__ __forceinline__ void tile_offsets(uint32_t (&off)[NP], int tid, int ldi, int k0, int seq_k) {
-    const int row = tid >> 4, col = (tid & 15) * 8;
-    constexpr int RSTEP = 64 / NP;
-#pragma unroll
-    for (int c = 0; c < NP; c++) {
-        int r = min(row + RSTEP * c, seq_k - 1 - k0);
-        off[c] = (uint32_t)(r * ldi + col) * 2u;
-    }
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
 template <int WAVES, bool CAUSAL, bool MASK>
@@ -172,8 +191,9 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
                int seq_q, int seq_k, int q_tiles, int total_work, int work_per_xcd,
                int kv_group, float scale_log2, const int *__restrict__ key_mask) {
-    extern __shared__ __align__(16) uint16_t lds[];     /* two stages of [K tile | V tile] */
-    constexpr int BM = 32 * WAVES, NP = 16 / WAVES;
+    extern __shared__ __align__(16) uint16_t lds[];     /* NSTAGE stages of [K tile | V tile] */
+    constexpr int BM = 32 * WAVES, NI = 32 / WAVES;
+    constexpr int NSTAGE = WAVES == 8 ? 3 : 2, AHEAD = NSTAGE - 1;     /* tiles in flight ahead of the one in use */
 
     /* XCD-aware numbering: hardware deals workgroups round-robin to the 8
      * XCDs, so id%8 is the XCD; give each XCD a contiguous slice of the
@@ -185,7 +205,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     if (CAUSAL) qt = q_tiles - 1 - qt;             /* longest rows first */
     const int kvh = head / kv_group;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;       /* 16x16 block: column li, row group lg */
     const int q0 = qt * BM, wq0 = q0 + wave * 32;
     const int qrow0 = wq0 + li, qrow1 = qrow0 + 16; /* this lane's two queries (query blocks 0 and 1) */
@@ -224,48 +244,63 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
      * V^T operand (dim block db, k-step ks): transpose read of a 4-key x 16-dim block per
      * 16-lane group; the lane supplies row 4lg + li/4 (+32ks, +16 for the second half)
      * and columns 4(li%4) (+16db), and receives the four keys of dim 16db + li. */
-    const int k_rd = li * KS + 8 * lg;
-    const int v_rd = K_TILE + (4 * lg + (li >> 2)) * VS + 4 * (li & 3);
-
-    /* Row offsets of this thread's 16 B pieces: one set for full tiles, one for
-     * the last tile (rows past seq_k redirected to the last valid row). */
-    const int last_k0 = (ntiles - 1) * BN;
-    uint32_t off_full[NP], off_last[NP];
-    tile_offsets(off_full, tid, ldi, 0, BN);
-    tile_offsets(off_last, tid, ldi, last_k0, seq_k);
-
-    /* ---- prologue: tile 0 -> stage 0, tile 1 -> registers. Tile indices past
-     * the end are clamped to the last tile: the copy is redundant but keeps the
-     * pipeline free of control flow. ---- */
-    TileRegs<NP> tile;
+    int k_rd[4], v_rd[8];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) k_rd[ks] = li * KS + 8 * ((4 * ks + lg) ^ swz(li));
     {
-        uint32_t off[NP];
+        const int vrow = 4 * lg + (li >> 2);
 #pragma unroll
-        for (int c = 0; c < NP; c++) off[c] = ntiles > 1 ? off_full[c] : off_last[c];
-        fetch_tile(tile, kbase, vbase, off);
-        store_tile(tile, lds, tid);
-        const int kn = min(BN, last_k0);
-#pragma unroll
-        for (int c = 0; c < NP; c++) off[c] = kn == last_k0 ? off_last[c] : off_full[c];
-        fetch_tile(tile, kbase + (size_t)kn * ldi, vbase + (size_t)kn * ldi, off);
+        for (int db = 0; db < 8; db++)
+            v_rd[db] = K_TILE + vrow * VS + 8 * ((2 * db + ((li & 3) >> 1)) ^ swz(vrow)) + 4 * (li & 1);
     }
-    __syncthreads();
 
+    /* This lane's source offsets inside a piece (bytes): row lane/16 of the piece, chunk by parity of the piece. */
+    const int last_k0 = (ntiles - 1) * BN;
+    uint32_t lane_off[2];
+#pragma unroll
+    for (int par = 0; par < 2; par++)
+        lane_off[par] = (uint32_t)((lane >> 4) * ldi + 8 * ((lane & 15) ^ swz(4 * par + (lane >> 4)))) * 2u;
+    auto request = [&](int tile_index, int stage) {      /* tile indices past the end repeat the last tile */
+        const int kn = min(tile_index * BN, last_k0);
+        const uint16_t *kt = kbase + (size_t)kn * ldi, *vt = vbase + (size_t)kn * ldi;
+        if (kn + BN <= seq_k) load_tile<NI>(lds + stage * STAGE, kt, vt, ldi, lane_off, wave);
+        else load_tile_clamped<NI>(lds + stage * STAGE, kt, vt, ldi, seq_k - 1 - kn, lane, wave);
+    };
+
+    /* The tile requests below are invisible to the compiler's own wait-count bookkeeping, so every
+     * load it does know about (Q) is completed here: the empty asm consumes the registers, which
+     * pins the loads and their wait before this point. Left to itself the compiler sinks the Q
+     * loads to the loop and re-waits for them in every iteration, which in fact waits for the
+     * newest tile requests. */
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            u32x4 t = __builtin_bit_cast(u32x4, qb[nb][ks]);
+            asm volatile("" : "+v"(t));
+            qb[nb][ks] = __builtin_bit_cast(bf16x8, t);
+        }
+
+    /* ---- prologue: tiles 0 .. AHEAD-1 on their way, tile 0 landed ---- */
+#pragma unroll
+    for (int t = 0; t < AHEAD; t++) request(t, t);
+    wait_vmcnt<NI * (AHEAD - 1)>();
+    __builtin_amdgcn_s_barrier();
+
+    int st_cur = 0, st_req = AHEAD;                      /* stage in use, stage to fill next */
     for (int it = 0; it < ntiles; it++) {
         const int k0 = it * BN;
-        uint16_t *cur = lds + (it & 1) * STAGE;
+        uint16_t *cur = lds + st_cur * STAGE;
 
-        /* tile it+1: registers -> the other stage (its last readers passed the barrier
-         * that ended the previous iteration); tile it+2: HBM -> registers */
-        store_tile(tile, lds + ((it + 1) & 1) * STAGE, tid);
-        {
-            const int kn = min(k0 + 2 * BN, last_k0);
-            const bool is_last = kn == last_k0;
-            uint32_t off[NP];
-#pragma unroll
-            for (int c = 0; c < NP; c++) off[c] = is_last ? off_last[c] : off_full[c];
-            fetch_tile(tile, kbase + (size_t)kn * ldi, vbase + (size_t)kn * ldi, off);
-        }
+        /* validity of the tile's keys: range / key mask as a wave-uniform 64-bit set (read before
+         * the tile requests below, so that waiting for it does not wait for them) */
+        unsigned long long valid = ~0ull;
+        if (k0 + BN > seq_k) valid = (1ull << (seq_k - k0)) - 1ull;
+        if (MASK) valid &= __ballot((k0 + lane < seq_k) && key_mask[min(k0 + lane, seq_k - 1)] != 0);
+
+        /* tile it+AHEAD: HBM/L2 -> the stage whose last readers passed the barrier that ended
+         * the previous iteration */
+        request(it + AHEAD, st_req);
 
         /* ---- S^T = K Q^T : 4 key blocks x 2 query blocks of 16x16, 4 k-steps of 32 dims.
          * All 16 A operands are requested from LDS up front so their latency
@@ -277,7 +312,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             for (int mb = 0; mb < 4; mb++)
 #pragma unroll
                 for (int ks = 0; ks < 4; ks++)
-                    ka[mb][ks] = *reinterpret_cast<const u32x4 *>(&cur[k_rd + 16 * mb * KS + 32 * ks]);
+                    ka[mb][ks] = *reinterpret_cast<const u32x4 *>(&cur[k_rd[ks] + 16 * mb * KS]);
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(1);
             const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -298,9 +333,6 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         /* s[mb][nb][r] is key k0 + 16mb + 4lg + r against query 16nb + li of the wave */
 
         /* ---- validity: range / key mask (wave-uniform 64-bit set), causal (per lane) ---- */
-        unsigned long long valid = ~0ull;
-        if (k0 + BN > seq_k) valid = (1ull << (seq_k - k0)) - 1ull;
-        if (MASK) valid &= __ballot((k0 + lane < seq_k) && key_mask[min(k0 + lane, seq_k - 1)] != 0);
         if (valid != ~0ull) {
             const unsigned long long mine = valid >> (4 * lg);
 #pragma unroll
@@ -371,7 +403,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             s16x4 lo[8], hi[8];
 #pragma unroll
             for (int db = 0; db < 8; db++) {
-                const uint16_t *vp = &cur[v_rd + 32 * ks * VS + 16 * db];
+                const uint16_t *vp = &cur[v_rd[db] + 32 * ks * VS];
                 lo[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp));
                 hi[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 16 * VS));
             }
@@ -388,8 +420,15 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             }
             __builtin_amdgcn_s_setprio(0);
         }
+        /* this wave's pieces of tile it+1 have landed; after the barrier everybody's have, and
+         * nobody reads stage st_cur any more */
+        wait_vmcnt<NI * (AHEAD - 1)>();
         lds_barrier();
+        st_cur = st_cur + 1 == NSTAGE ? 0 : st_cur + 1;
+        st_req = st_req + 1 == NSTAGE ? 0 : st_req + 1;
     }
+
+    wait_vmcnt<0>();       /* the repeated requests of the last iterations must land before the LDS is given back */
 
     /* ---- normalise and store: the lane holds dims 16db + 4lg + {0..3} of its two queries ---- */
 #pragma unroll
@@ -410,7 +449,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     }
 }
 
-constexpr size_t LDS_BYTES = 2 * STAGE * sizeof(uint16_t);
+template <int W> constexpr size_t lds_bytes() { return (W == 8 ? 3 : 2) * STAGE * sizeof(uint16_t); }
 constexpr int CUS = 256;
 
 template <int W, bool C, bool M>
@@ -420,14 +459,14 @@ int launch(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd128<W, C, M>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes<W>());
         if (e != hipSuccess) return (int)e;
         configured = true;
     }
     const int q_tiles = (seq_q + 32 * W - 1) / (32 * W);
     const int total = q_tiles * heads;
     const int per_xcd = (total + XCDS - 1) / XCDS;
-    hipLaunchKernelGGL((k_fa_fwd_hd128<W, C, M>), dim3(per_xcd * XCDS), dim3(64 * W), LDS_BYTES, st, out, ldo,
+    hipLaunchKernelGGL((k_fa_fwd_hd128<W, C, M>), dim3(per_xcd * XCDS), dim3(64 * W), lds_bytes<W>(), st, out, ldo,
                        q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, heads / kv_heads,
                        scale * 1.4426950408889634f, key_mask);
     return (int)hipGetLastError();
@@ -452,10 +491,20 @@ extern "C" int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uin
                                  int seq_k, int heads, int kv_heads, float scale, int causal,
                                  const int *key_mask) {
     hipStream_t st = (hipStream_t)stream;
-    /* 256 queries per workgroup halve the K/V traffic from L2 and the LDS writes per query;
-     * 128 give twice the workgroups when the problem is too small to fill the CUs. */
+    /* 256 queries per workgroup halve the K/V traffic from L2 per query, but one such workgroup
+     * fills a CU, so the grid runs in rounds of 256 and a badly filled last round is expensive:
+     * they are used when the rounds are at least 80 % full. 128 queries (two workgroups per CU)
+     * otherwise. A workgroup walks its key tiles one after the other, about 2 us each, so a short
+     * sequence is bound by that latency and wants many small workgroups: 64 or 32 queries when
+     * the larger shapes would leave CUs without work (measured on 24 heads, 256 .. 4608 tokens). */
+    const long units = (long)((seq_q + 31) / 32) * heads;          /* waves of 32 queries */
     const long wg256 = (long)((seq_q + 255) / 256) * heads;
-    if (wg256 >= CUS)
+    const long rounds = (wg256 + CUS - 1) / CUS;
+    if (units >= 576 && 5 * wg256 >= 4 * rounds * CUS)
         return launch_w<8>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
-    return launch_w<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
+    if (units >= 576)
+        return launch_w<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
+    if (units >= 256)
+        return launch_w<2>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
+    return launch_w<1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
 }

@@ -112,6 +112,32 @@ def test_c2_full_size_sampled_rows_and_properties(dev, orc):
     assert_close(got3, want, "C2 constant V")
 
 
+@pytest.mark.parametrize("seq,heads,kv,causal,masked", [
+    (200, 6, 6, False, False), (200, 6, 2, True, True),              # 32-query workgroups (one wave)
+    (600, 16, 4, False, True), (600, 16, 16, True, False),           # 64-query workgroups
+    (1300, 16, 16, False, False), (1300, 16, 8, True, True),         # 128-query workgroups
+    (2100, 24, 8, False, True), (2100, 24, 24, True, False),         # 256-query workgroups
+])
+def test_every_workgroup_width(dev, orc, seq, heads, kv, causal, masked):
+    """The launcher picks 32, 64, 128 or 256 queries per workgroup from the problem size; each
+    width is its own instantiation of the kernel (pieces of a key tile per wave, LDS stages).
+    Sampled rows against the oracle, including the rows around every workgroup boundary."""
+    rng = np.random.default_rng(seq + heads)
+    ldi = (heads + 2 * kv) * 128
+    buf = O.f32_to_bf16(rng.standard_normal((seq, ldi)).astype(np.float32))
+    mask = None
+    if masked:
+        mask = (rng.random(seq) < 0.7).astype(np.int32)
+        mask[0] = 1                                                     # every causal row keeps a valid key
+    case = W._case(buf=buf, heads=heads, kv_heads=kv, causal=causal, key_mask=mask)
+    case["ldo"] = heads * 128
+    got, kernel = gpu_attention(dev, case)
+    assert kernel == "fa_hd128"
+    rows = np.unique(np.r_[sample_rows(seq, n=24, seed=seq), [31, 32, 63, 64, 255, 256 % seq, seq - 33, seq - 32]]).astype(np.int32)
+    rows = rows[(rows >= 0) & (rows < seq)]
+    assert_close(got[rows], cpu_attention(orc, case, rows=rows), f"seq {seq} heads {heads}/{kv}")
+
+
 def test_c5_full_size_sampled_rows(dev, orc):
     case = after_norm_rope(dev, W.c5())           # 12800 tokens
     got, kernel = gpu_attention(dev, case)
