@@ -267,6 +267,18 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         else load_tile_clamped<NI>(lds + stage * STAGE, kt, vt, ldi, seq_k - 1 - kn, lane, wave);
     };
 
+    /* The key mask as one 64-bit word per key tile, kept in LDS behind the stages: built once here,
+     * so that the loop has no global load of its own (a load there would be waited for with
+     * vmcnt(0), i.e. together with the newest tile requests). Keys past seq_k count as masked. */
+    unsigned long long *mask_words = reinterpret_cast<unsigned long long *>(lds + NSTAGE * STAGE);
+    if (MASK) {
+        for (int t = wave; t < ntiles; t += WAVES) {
+            const int key = t * BN + lane;
+            const unsigned long long word = __ballot(key < seq_k && key_mask[min(key, seq_k - 1)] != 0);
+            if (lane == 0) mask_words[t] = word;
+        }
+    }
+
     /* The tile requests below are invisible to the compiler's own wait-count bookkeeping, so every
      * load it does know about (Q) is completed here: the empty asm consumes the registers, which
      * pins the loads and their wait before this point. Left to itself the compiler sinks the Q
@@ -285,7 +297,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 #pragma unroll
     for (int t = 0; t < AHEAD; t++) request(t, t);
     wait_vmcnt<NI * (AHEAD - 1)>();
-    __builtin_amdgcn_s_barrier();
+    lds_barrier();                                       /* also publishes the key-mask words */
 
     int st_cur = 0, st_req = AHEAD;                      /* stage in use, stage to fill next */
     for (int it = 0; it < ntiles; it++) {
@@ -296,7 +308,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
          * the tile requests below, so that waiting for it does not wait for them) */
         unsigned long long valid = ~0ull;
         if (k0 + BN > seq_k) valid = (1ull << (seq_k - k0)) - 1ull;
-        if (MASK) valid &= __ballot((k0 + lane < seq_k) && key_mask[min(k0 + lane, seq_k - 1)] != 0);
+        if (MASK) valid &= mask_words[it];
 
         /* tile it+AHEAD: HBM/L2 -> the stage whose last readers passed the barrier that ended
          * the previous iteration */
@@ -449,7 +461,8 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     }
 }
 
-template <int W> constexpr size_t lds_bytes() { return (W == 8 ? 3 : 2) * STAGE * sizeof(uint16_t); }
+template <int W> constexpr size_t stage_bytes() { return (W == 8 ? 3 : 2) * STAGE * sizeof(uint16_t); }
+constexpr size_t LDS_MAX = 160 * 1024;
 constexpr int CUS = 256;
 
 template <int W, bool C, bool M>
@@ -459,14 +472,17 @@ int launch(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd128<W, C, M>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes<W>());
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
         if (e != hipSuccess) return (int)e;
         configured = true;
     }
     const int q_tiles = (seq_q + 32 * W - 1) / (32 * W);
     const int total = q_tiles * heads;
     const int per_xcd = (total + XCDS - 1) / XCDS;
-    hipLaunchKernelGGL((k_fa_fwd_hd128<W, C, M>), dim3(per_xcd * XCDS), dim3(64 * W), lds_bytes<W>(), st, out, ldo,
+    /* the stages, and for a key mask one 64-bit word per key tile behind them */
+    const size_t lds_bytes = stage_bytes<W>() + (M ? 8 * (size_t)((seq_k + BN - 1) / BN) : 0);
+    if (lds_bytes > LDS_MAX) return (int)hipErrorInvalidValue;       /* the caller keeps masked seq_k below the limit */
+    hipLaunchKernelGGL((k_fa_fwd_hd128<W, C, M>), dim3(per_xcd * XCDS), dim3(64 * W), lds_bytes, st, out, ldo,
                        q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, heads / kv_heads,
                        scale * 1.4426950408889634f, key_mask);
     return (int)hipGetLastError();

@@ -205,7 +205,7 @@ void iris_dev_attention(uint16_t *out, int ldo,
     int mfma_ok = seq_k > 0 && scale > 0.0f && ldi % 8 == 0 && ldo % 4 == 0 &&
                   aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out, 8);
     int err;
-    if (mfma_ok && head_dim == 128) {
+    if (mfma_ok && head_dim == 128 && (!key_mask || seq_k <= IRIS_FA_MAX_MASKED_KEYS)) {
         g_last_kernel = "fa_hd128";
         err = iris_hip_fa_hd128(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads,
                                 scale, causal != 0, key_mask);

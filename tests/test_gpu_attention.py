@@ -138,6 +138,40 @@ def test_every_workgroup_width(dev, orc, seq, heads, kv, causal, masked):
     assert_close(got[rows], cpu_attention(orc, case, rows=rows), f"seq {seq} heads {heads}/{kv}")
 
 
+def test_very_long_masked_key_sequence_takes_the_generic_kernel(dev, orc):
+    """The matrix-core kernel keeps the key mask in LDS, one bit per key, which bounds a masked
+    seq_k at 500000; beyond that the call must still be answered (by the generic kernel)."""
+    seq_k, seq_q, ldi = 500_001, 2, 256                    # q in columns 0..127 of the first rows, k = v in 128..255
+    rng = np.random.default_rng(77)
+    buf = O.f32_to_bf16((rng.integers(-8, 9, (seq_k, ldi)) / 8).astype(np.float32))
+    mask = (rng.random(seq_k) < 0.5).astype(np.int32)
+    out, kernel = dev.attention(buf, ldi, 0, 128, 128, seq_q, seq_k, 1, 1, 128, 0.09, False, mask, ldo=128)
+    assert kernel == "attention_generic"
+    want = orc.attention_bf16(buf, ldi, 0, 128, 128, seq_q, seq_k, 1, 1, 128, 0.09, False, mask)
+    assert_close(O.bf16_to_f32(out), want, "500001 masked keys")
+    # one key fewer than the limit still runs on the matrix cores
+    out, kernel = dev.attention(buf, ldi, 0, 128, 128, seq_q, 499_968, 1, 1, 128, 0.09, False, mask[:499_968], ldo=128)
+    assert kernel == "fa_hd128"
+    want = orc.attention_bf16(buf, ldi, 0, 128, 128, seq_q, 499_968, 1, 1, 128, 0.09, False, mask[:499_968])
+    assert_close(O.bf16_to_f32(out), want, "499968 masked keys")
+
+
+def test_long_sequence_offsets(dev, orc):
+    """40000 tokens: row offsets beyond 2^31 bytes into the fused buffer must not wrap."""
+    seq, heads = 40_000, 2
+    ldi = 3 * heads * 128 + 26_000                           # wide rows: 40000 x 26768 x 2 B = 2.1 GB
+    ldi -= ldi % 8
+    rng = np.random.default_rng(9)
+    buf = np.zeros((seq, ldi), np.uint16)
+    buf[:, :3 * heads * 128] = O.f32_to_bf16(rng.standard_normal((seq, 3 * heads * 128)).astype(np.float32))
+    case = W._case(buf=buf, heads=heads, kv_heads=heads)
+    case["ldo"] = heads * 128
+    got, kernel = gpu_attention(dev, case)
+    assert kernel == "fa_hd128"
+    rows = np.array([0, 1, 255, 19_999, 39_000, 39_999], np.int32)
+    assert_close(got[rows], cpu_attention(orc, case, rows=rows), "40000 tokens, 2.1 GB of rows")
+
+
 def test_c5_full_size_sampled_rows(dev, orc):
     case = after_norm_rope(dev, W.c5())           # 12800 tokens
     got, kernel = gpu_attention(dev, case)
