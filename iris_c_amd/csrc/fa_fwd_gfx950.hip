@@ -315,32 +315,35 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         request(it + AHEAD, st_req);
 
         /* ---- S^T = K Q^T : 4 key blocks x 2 query blocks of 16x16, 4 k-steps of 32 dims.
-         * All 16 A operands are requested from LDS up front so their latency
-         * overlaps instead of gating every MFMA; each feeds two MFMAs. ---- */
+         * Software pipeline over the k-steps: the four A operands of step ks+1 are requested from
+         * LDS before the eight MFMAs of step ks are issued, so that the LDS serves reads all the
+         * time the matrix core works instead of in one burst from all waves that the MFMAs then
+         * wait for. Each operand feeds two MFMAs. ---- */
         f32x4 s[4][2];
         {
-            u32x4 ka[4][4];
+            u32x4 ka[2][4];                                /* two k-steps in flight */
+            auto read_k = [&](int ks) {
 #pragma unroll
-            for (int mb = 0; mb < 4; mb++)
-#pragma unroll
-                for (int ks = 0; ks < 4; ks++)
-                    ka[mb][ks] = *reinterpret_cast<const u32x4 *>(&cur[k_rd[ks] + 16 * mb * KS]);
+                for (int mb = 0; mb < 4; mb++)
+                    ka[ks & 1][mb] = *reinterpret_cast<const u32x4 *>(&cur[k_rd[ks] + 16 * mb * KS]);
+            };
+            read_k(0);
             __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_setprio(1);
             const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int mb = 0; mb < 4; mb++)
-#pragma unroll
-                for (int nb = 0; nb < 2; nb++)
-                    s[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[mb][0]), qb[nb][0], zero, 0, 0, 0);
-#pragma unroll
-            for (int ks = 1; ks < 4; ks++)
+            for (int ks = 0; ks < 4; ks++) {
+                if (ks < 3) read_k(ks + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                
 #pragma unroll
                 for (int mb = 0; mb < 4; mb++)
 #pragma unroll
                     for (int nb = 0; nb < 2; nb++)
-                        s[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[mb][ks]), qb[nb][ks], s[mb][nb], 0, 0, 0);
-            __builtin_amdgcn_s_setprio(0);
+                        s[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[ks & 1][mb]), qb[nb][ks],
+                                                                            ks == 0 ? zero : s[mb][nb], 0, 0, 0);
+                
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         /* s[mb][nb][r] is key k0 + 16mb + 4lg + r against query 16nb + li of the wave */
 
@@ -408,29 +411,42 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             }
         }
 
-        /* ---- O^T += V^T P^T : 2 k-steps of 32 keys x 8 dim blocks x 2 query blocks; the V^T
-         * operands of a k-step are requested together ---- */
+        /* ---- O^T += V^T P^T : 2 k-steps of 32 keys x 8 dim blocks x 2 query blocks, pipelined the
+         * same way in four groups of four dim blocks: the V^T operands of the next group are
+         * requested before the MFMAs of this one ---- */
+        {
+            s16x4 lo[2][4], hi[2][4];                      /* two groups in flight */
+            auto read_v = [&](int g) {                     /* group g: k-step g / 2, dim blocks 4 (g % 2) .. +3 */
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
-            s16x4 lo[8], hi[8];
-#pragma unroll
-            for (int db = 0; db < 8; db++) {
-                const uint16_t *vp = &cur[v_rd[db] + 32 * ks * VS];
-                lo[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp));
-                hi[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 16 * VS));
-            }
+                for (int d = 0; d < 4; d++) {
+                    const uint16_t *vp = &cur[v_rd[4 * (g & 1) + d] + 32 * (g >> 1) * VS];
+                    lo[g & 1][d] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp));
+                    hi[g & 1][d] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 16 * VS));
+                }
+            };
+            read_v(0);
             __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_setprio(1);
-            const bf16x8 pb0 = __builtin_bit_cast(bf16x8, pw[ks][0]), pb1 = __builtin_bit_cast(bf16x8, pw[ks][1]);
-            l_acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb0, l_acc[0], 0, 0, 0);
-            l_acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb1, l_acc[1], 0, 0, 0);
 #pragma unroll
-            for (int db = 0; db < 8; db++) {
-                s16x8 both = __builtin_shufflevector(lo[db], hi[db], 0, 1, 2, 3, 4, 5, 6, 7);
-                o[db][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb0, o[db][0], 0, 0, 0);
-                o[db][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb1, o[db][1], 0, 0, 0);
+            for (int g = 0; g < 4; g++) {
+                if (g < 3) read_v(g + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                
+                const int ks = g >> 1;
+                const bf16x8 pb0 = __builtin_bit_cast(bf16x8, pw[ks][0]), pb1 = __builtin_bit_cast(bf16x8, pw[ks][1]);
+                if ((g & 1) == 0) {
+                    l_acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb0, l_acc[0], 0, 0, 0);
+                    l_acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb1, l_acc[1], 0, 0, 0);
+                }
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+                    const int db = 4 * (g & 1) + d;
+                    s16x8 both = __builtin_shufflevector(lo[g & 1][d], hi[g & 1][d], 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[db][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb0, o[db][0], 0, 0, 0);
+                    o[db][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb1, o[db][1], 0, 0, 0);
+                }
+                
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_s_setprio(0);
         }
         /* this wave's pieces of tile it+1 have landed; after the barrier everybody's have, and
          * nobody reads stage st_cur any more */
