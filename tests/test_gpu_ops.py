@@ -214,3 +214,31 @@ def test_upsample2x(dev, orc, h, w, c):
     dimg, dout = dev.put(img), dev.alloc(4 * h * w * c * 4)
     got = run(dev, lambda: dev.lib.iris_dev_upsample2x(dout, dimg, h, w, c), [(dout, (4 * h * w, c), np.float32)])
     np.testing.assert_array_equal(got, orc.dev_upsample2x(img, h, w))
+
+
+def test_cleanup_and_second_init(dev, orc):
+    """iris_dev_cleanup releases the stream and every private scratch (convolution patches, group-norm
+    partials, table staging, the GEMM library's handle and workspace); a later iris_dev_init must bring
+    all of it back: the reference's program initialises once per process, a test harness may not."""
+    lib = dev.lib
+    rows, k, out = 64, 128, 64
+    x, W = O.f32_to_bf16(rnd((rows, k), 1)), O.f32_to_bf16(rnd((out, k), 2, 0.05))
+    want = orc.dev_linear(x, W)
+
+    def linear_once():
+        dx, dW, dy = dev.put(x), dev.put(W), dev.alloc(rows * out * 4)
+        return run(dev, lambda: lib.iris_dev_linear_f32(dy, dx, dW, rows, k, out), [(dy, (rows, out), np.float32)])
+
+    np.testing.assert_allclose(linear_once(), want, atol=1e-4)
+    lib.iris_dev_cleanup()
+    assert lib.iris_dev_available() == 0
+    assert lib.iris_dev_alloc(16) is None                    # refused, not crashed
+    lib.iris_dev_last_error()
+    assert lib.iris_dev_init() == 1 and lib.iris_dev_available() == 1
+    np.testing.assert_allclose(linear_once(), want, atol=1e-4)
+    assert dev.dev.last_kernel() == "linear_hipblaslt"       # the library was opened again
+    # an operator with private scratch after the re-init
+    img, gamma, beta = rnd((100, 8), 5), 1 + rnd(8, 1, 0.1), rnd(8, 2, 0.1)
+    dimg, dg, db, dout = dev.put(img), dev.put(gamma), dev.put(beta), dev.alloc(100 * 8 * 4)
+    got = run(dev, lambda: lib.iris_dev_group_norm(dout, dimg, dg, db, 100, 8, 2, 1e-6, 0), [(dout, (100, 8), np.float32)])
+    np.testing.assert_allclose(got, orc.dev_group_norm(img, gamma, beta, 2, 1e-6, 0), atol=2e-5)
