@@ -23,10 +23,11 @@
  * ones are taken when the problem has too few queries to give every CU a
  * large workgroup: a workgroup walks its key tiles one after the other, so a
  * short sequence is bound by that latency and wants many small workgroups.
- * Keys/values stream through LDS in tiles of 64 keys, 3 stages (2 below 8
+ * Keys/values stream through LDS in tiles of 64 keys, 4 stages (2 below 8
  * waves), and they go there directly: global_load_lds_dwordx4 copies
- * HBM/L2 -> LDS without passing through registers, two tiles ahead of the
- * one in use; one barrier per tile. Every wave reads the whole K and V tile,
+ * HBM/L2 -> LDS without passing through registers, one group of tiles
+ * (two tiles, one below 8 waves) ahead of the group in use; one barrier per
+ * group. Every wave reads the whole K and V tile,
  * so 256 queries per workgroup mean half the L2 -> LDS traffic per query of
  * 128.
  *
@@ -193,7 +194,11 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                int kv_group, float scale_log2, const int *__restrict__ key_mask) {
     extern __shared__ __align__(16) uint16_t lds[];     /* NSTAGE stages of [K tile | V tile] */
     constexpr int BM = 32 * WAVES, NI = 32 / WAVES;
-    constexpr int NSTAGE = WAVES == 8 ? 3 : 2, AHEAD = NSTAGE - 1;     /* tiles in flight ahead of the one in use */
+    /* Key tiles between two barriers. Two for the 8-wave shape (one workgroup per CU, so the LDS
+     * has room for four stages): the waves of a workgroup then only meet every other tile, and
+     * the faster ones do not stand at a barrier while the slower ones finish every single tile. */
+    constexpr int GROUP = WAVES == 8 ? 2 : 1;
+    constexpr int NSTAGE = 2 * GROUP;                    /* the group in use and the group on its way */
 
     /* XCD-aware numbering: hardware deals workgroups round-robin to the 8
      * XCDs, so id%8 is the XCD; give each XCD a contiguous slice of the
@@ -293,26 +298,29 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             qb[nb][ks] = __builtin_bit_cast(bf16x8, t);
         }
 
-    /* ---- prologue: tiles 0 .. AHEAD-1 on their way, tile 0 landed ---- */
+    /* ---- prologue: the first group of tiles landed ---- */
 #pragma unroll
-    for (int t = 0; t < AHEAD; t++) request(t, t);
-    wait_vmcnt<NI * (AHEAD - 1)>();
+    for (int t = 0; t < GROUP; t++) request(t, t);
+    wait_vmcnt<0>();
     lds_barrier();                                       /* also publishes the key-mask words */
 
-    int st_cur = 0, st_req = AHEAD;                      /* stage in use, stage to fill next */
-    for (int it = 0; it < ntiles; it++) {
+    for (int g0 = 0, half = 0; g0 < ntiles; g0 += GROUP, half ^= 1) {
+        /* the next group: HBM/L2 -> the stages whose last readers passed the barrier that ended the
+         * previous group; it has this whole group's time to land */
+#pragma unroll
+        for (int t = 0; t < GROUP; t++) request(g0 + GROUP + t, (half ^ 1) * GROUP + t);
+#pragma unroll
+      for (int h = 0; h < GROUP; h++) {
+        const int it = g0 + h;
+        if (it >= ntiles) break;                         /* wave-uniform */
         const int k0 = it * BN;
-        uint16_t *cur = lds + st_cur * STAGE;
+        uint16_t *cur = lds + (half * GROUP + h) * STAGE;
 
         /* validity of the tile's keys: range / key mask as a wave-uniform 64-bit set (read before
          * the tile requests below, so that waiting for it does not wait for them) */
         unsigned long long valid = ~0ull;
         if (k0 + BN > seq_k) valid = (1ull << (seq_k - k0)) - 1ull;
         if (MASK) valid &= mask_words[it];
-
-        /* tile it+AHEAD: HBM/L2 -> the stage whose last readers passed the barrier that ended
-         * the previous iteration */
-        request(it + AHEAD, st_req);
 
         /* ---- S^T = K Q^T : 4 key blocks x 2 query blocks of 16x16, 4 k-steps of 32 dims.
          * Software pipeline over the k-steps: the four A operands of step ks+1 are requested from
@@ -448,15 +456,14 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        /* this wave's pieces of tile it+1 have landed; after the barrier everybody's have, and
-         * nobody reads stage st_cur any more */
-        wait_vmcnt<NI * (AHEAD - 1)>();
+      }
+        /* this wave's pieces of the next group have landed; after the barrier everybody's have, and
+         * nobody reads the stages of this group any more */
+        wait_vmcnt<0>();
         lds_barrier();
-        st_cur = st_cur + 1 == NSTAGE ? 0 : st_cur + 1;
-        st_req = st_req + 1 == NSTAGE ? 0 : st_req + 1;
     }
 
-    wait_vmcnt<0>();       /* the repeated requests of the last iterations must land before the LDS is given back */
+    wait_vmcnt<0>();       /* nothing may still be on its way into the LDS when it is given back (the loop ends with this wait too) */
 
     /* ---- normalise and store: the lane holds dims 16db + 4lg + {0..3} of its two queries ---- */
 #pragma unroll
@@ -477,7 +484,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     }
 }
 
-template <int W> constexpr size_t stage_bytes() { return (W == 8 ? 3 : 2) * STAGE * sizeof(uint16_t); }
+template <int W> constexpr size_t stage_bytes() { return (W == 8 ? 4 : 2) * STAGE * sizeof(uint16_t); }
 constexpr size_t LDS_MAX = 160 * 1024;
 constexpr int CUS = 256;
 

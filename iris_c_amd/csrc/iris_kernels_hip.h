@@ -31,7 +31,7 @@ int iris_hip_norm_rope_generic(void *stream, uint16_t *x, int ld, const float *w
  * aligned, ldi % 8 == 0, out 8-byte aligned, ldo % 4 == 0, scale > 0,
  * heads % kv_heads == 0, seq_q > 0, seq_k > 0, and with a key mask
  * seq_k <= IRIS_FA_MAX_MASKED_KEYS (the mask is kept in LDS as one bit per key). */
-#define IRIS_FA_MAX_MASKED_KEYS 500000
+#define IRIS_FA_MAX_MASKED_KEYS 250000
 int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uint16_t *q,
                       const uint16_t *k, const uint16_t *v, int ldi, int seq_q, int seq_k,
                       int heads, int kv_heads, float scale, int causal, const int *key_mask);

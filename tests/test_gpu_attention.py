@@ -140,20 +140,20 @@ def test_every_workgroup_width(dev, orc, seq, heads, kv, causal, masked):
 
 def test_very_long_masked_key_sequence_takes_the_generic_kernel(dev, orc):
     """The matrix-core kernel keeps the key mask in LDS, one bit per key, which bounds a masked
-    seq_k at 500000; beyond that the call must still be answered (by the generic kernel)."""
-    seq_k, seq_q, ldi = 500_001, 2, 256                    # q in columns 0..127 of the first rows, k = v in 128..255
+    seq_k at 250000; beyond that the call must still be answered (by the generic kernel)."""
+    seq_k, seq_q, ldi = 250_001, 2, 256                    # q in columns 0..127 of the first rows, k = v in 128..255
     rng = np.random.default_rng(77)
     buf = O.f32_to_bf16((rng.integers(-8, 9, (seq_k, ldi)) / 8).astype(np.float32))
     mask = (rng.random(seq_k) < 0.5).astype(np.int32)
     out, kernel = dev.attention(buf, ldi, 0, 128, 128, seq_q, seq_k, 1, 1, 128, 0.09, False, mask, ldo=128)
     assert kernel == "attention_generic"
     want = orc.attention_bf16(buf, ldi, 0, 128, 128, seq_q, seq_k, 1, 1, 128, 0.09, False, mask)
-    assert_close(O.bf16_to_f32(out), want, "500001 masked keys")
+    assert_close(O.bf16_to_f32(out), want, "250001 masked keys")
     # one key fewer than the limit still runs on the matrix cores
-    out, kernel = dev.attention(buf, ldi, 0, 128, 128, seq_q, 499_968, 1, 1, 128, 0.09, False, mask[:499_968], ldo=128)
+    out, kernel = dev.attention(buf, ldi, 0, 128, 128, seq_q, 249_984, 1, 1, 128, 0.09, False, mask[:249_984], ldo=128)
     assert kernel == "fa_hd128"
-    want = orc.attention_bf16(buf, ldi, 0, 128, 128, seq_q, 499_968, 1, 1, 128, 0.09, False, mask[:499_968])
-    assert_close(O.bf16_to_f32(out), want, "499968 masked keys")
+    want = orc.attention_bf16(buf, ldi, 0, 128, 128, seq_q, 249_984, 1, 1, 128, 0.09, False, mask[:249_984])
+    assert_close(O.bf16_to_f32(out), want, "249984 masked keys")
 
 
 def test_long_sequence_offsets(dev, orc):
