@@ -149,16 +149,45 @@ __device__ __forceinline__ uint32_t lds_address(const uint16_t *p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
 }
 
+/* a pointer the compiler must keep in scalar registers (it is wave-uniform, but selected at run time) */
+__device__ __forceinline__ const uint16_t *scalar_ptr(const uint16_t *p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const uint16_t *)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
 template <int NI>
 __device__ __forceinline__ void load_tile(uint16_t *stage, const uint16_t *kt, const uint16_t *vt, int ldi,
                                           const uint32_t (&lane_off)[2], int wave) {
+    if constexpr (NI <= 8) {
 #pragma unroll
-    for (int j = 0; j < NI; j++) {
-        const int g = wave * NI + j;                       /* wave-uniform */
-        const uint16_t *src = (g < 16 ? kt : vt) + (size_t)(4 * (g & 15)) * ldi;      /* first row of the piece */
-        const uint16_t *dst = stage + (g < 16 ? 0 : K_TILE) + 4 * (g & 15) * KS;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                     ::"s"(lds_address(dst)), "v"(lane_off[g & 1]), "s"(src) : "memory");
+        for (int j = 0; j < NI; j++) {
+            const int g = wave * NI + j;                       /* wave-uniform */
+            const uint16_t *src = (g < 16 ? kt : vt) + (size_t)(4 * (g & 15)) * ldi;      /* first row of the piece */
+            const uint16_t *dst = stage + (g < 16 ? 0 : K_TILE) + 4 * (g & 15) * KS;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         ::"s"(lds_address(dst)), "v"(lane_off[g & 1]), "s"(src) : "memory");
+        }
+    } else {
+        /* 16 or 32 pieces per wave (2 waves: one takes K, the other V; 1 wave: K then V). Source
+         * pointer and LDS address are advanced from piece to piece, and the empty asm hides the
+         * running values from the compiler: computed independently, the 32 pointers and addresses
+         * become invariants of the tile loop and spill out of the scalar registers. */
+#pragma unroll
+        for (int part = 0; part < NI / 16; part++) {
+            const bool is_v = wave * NI + 16 * part >= 16;
+            const uint16_t *src = scalar_ptr(is_v ? vt : kt);
+            uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(stage + (is_v ? K_TILE : 0)));
+            const size_t step = 4 * (size_t)ldi;
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                             ::"s"(dst), "v"(lane_off[j & 1]), "s"(src) : "memory");
+                src += step;
+                dst += 4 * KS * 2;
+                asm volatile("" : "+s"(src), "+s"(dst));
+            }
+        }
     }
 }
 
