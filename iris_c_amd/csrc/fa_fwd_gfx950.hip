@@ -334,10 +334,6 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     lds_barrier();                                       /* also publishes the key-mask words */
 
     for (int g0 = 0, half = 0; g0 < ntiles; g0 += GROUP, half ^= 1) {
-        /* the next group: HBM/L2 -> the stages whose last readers passed the barrier that ended the
-         * previous group; it has this whole group's time to land */
-#pragma unroll
-        for (int t = 0; t < GROUP; t++) request(g0 + GROUP + t, (half ^ 1) * GROUP + t);
 #pragma unroll
       for (int h = 0; h < GROUP; h++) {
         const int it = g0 + h;
@@ -381,6 +377,16 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                 
                 __builtin_amdgcn_sched_barrier(0);
             }
+        }
+        /* The next group: HBM/L2 -> the stages whose last readers passed the barrier that ended the
+         * previous group. Requested here, behind the first tile's QK product, and not right after
+         * the barrier: there every wave would issue its requests before its first operand read,
+         * with the matrix cores of the whole CU idle meanwhile. It still has the rest of the
+         * group's time to land. */
+        if (h == 0) {
+#pragma unroll
+            for (int t = 0; t < GROUP; t++) request(g0 + GROUP + t, (half ^ 1) * GROUP + t);
+            __builtin_amdgcn_sched_barrier(0);
         }
         /* s[mb][nb][r] is key k0 + 16mb + 4lg + r against query 16nb + li of the wave */
 
