@@ -14,7 +14,9 @@ OUT    = iris_c_amd/libiris_dev.so
 # Packed-f32 instruction selection is switched off for all device code.
 HIPFLAGS = -O3 --offload-arch=$(GPU_ARCH) -fPIC -std=c++17 -Xclang -target-feature -Xclang -packed-fp32-ops \
            -I$(CSRC) -Iinclude
-CFLAGS   = -O2 -fPIC -Wall -Wextra -std=c11 -I$(CSRC) -Iinclude -I$(ROCM_HOME)/include
+# gcc/g++ read the HIP runtime's host headers: they want the platform named on the command line
+HOSTDEFS = -D__HIP_PLATFORM_AMD__=1
+CFLAGS   = -O2 -fPIC -Wall -Wextra -std=c11 $(HOSTDEFS) -I$(CSRC) -Iinclude -I$(ROCM_HOME)/include
 
 HIP_SRCS = $(CSRC)/qknorm_rope.hip $(CSRC)/fa_fwd_gfx950.hip $(CSRC)/fa_fwd_sliced_gfx950.hip $(CSRC)/attn_generic.hip \
            $(CSRC)/ew_norm_ops.hip $(CSRC)/gemm_conv_gfx950.hip $(CSRC)/rope_tables.hip
@@ -49,7 +51,7 @@ $(CSRC)/iris_rope_tables.o: $(CSRC)/iris_rope_tables.c $(HOST_HDRS)
 
 # glue to the vendor GEMM library: host C++ only; the library itself is opened with dlopen at run time
 $(CSRC)/linear_hipblaslt.o: $(CSRC)/linear_hipblaslt.cpp $(CSRC)/iris_kernels_hip.h
-	$(CXX) -O2 -fPIC -Wall -Wextra -std=c++17 -I$(CSRC) -I$(ROCM_HOME)/include -c $< -o $@
+	$(CXX) -O2 -fPIC -Wall -Wextra -std=c++17 $(HOSTDEFS) -I$(CSRC) -I$(ROCM_HOME)/include -c $< -o $@
 
 $(OUT): $(HIP_OBJS) $(CSRC)/iris_rocm.o $(CSRC)/iris_rope_tables.o $(CSRC)/linear_hipblaslt.o
 	$(HIPCC) --offload-arch=$(GPU_ARCH) -shared -o $@ $^ -L$(ROCM_HOME)/lib -lamdhip64 -lm -ldl

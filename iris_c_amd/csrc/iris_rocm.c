@@ -11,7 +11,6 @@
  * the device is missing or the library was not initialised, the entries
  * report the error and leave the output untouched.
  */
-#define __HIP_PLATFORM_AMD__ 1
 #include <hip/hip_runtime_api.h>
 
 #include <stdio.h>

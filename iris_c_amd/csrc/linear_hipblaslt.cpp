@@ -18,7 +18,6 @@
  * One plan (descriptors + the heuristic's first algorithm) is kept per
  * distinct (out, rows, in, output type); a model uses a handful.
  */
-#define __HIP_PLATFORM_AMD__ 1
 #include <hip/hip_runtime_api.h>
 #include <hipblaslt/hipblaslt.h>
 
