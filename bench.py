@@ -6,17 +6,27 @@ sequence: fused per-head RMSNorm + RoPE on Q, on K, then joint attention
 (reference iris_transformer_flux.c:3834-3839), on the 24 heads x 128,
 512 text + 4096 image token configuration, bf16, inputs resident in HBM.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-shapes]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle-ms T] [--no-cpu] [--no-shapes]
 
 Prints ONE JSON line. `value` is attention TFLOP/s over the whole step
 (algorithmic attention FLOPs / wall time of the triple). `roofline` is the
-attention kernel alone, timed with HIP events on the library's stream.
-`norm_rope` reports the bandwidth-bound kernel the same way. `shapes` lists
+attention kernel alone, timed with HIP events on the library's stream around
+the attention launch of every step. `norm_rope` reports the bandwidth-bound
+kernel over back-to-back launches. `shapes` lists
 latency / TFLOP/s / GB/s for every benchmark configuration, `other_ops` the
 other device operators at this configuration's shapes, `rope_tables` the
 time to build one forward pass's rotary tables (host builder + upload, and
 the device generator). `cpu_baseline`
 times the reference's BLAS-build CPU structure on this host's cores.
+
+Clock settling: after idle the GPU's power management takes tens of
+milliseconds of sustained load to reach its steady clocks; the same
+attention launch measures 0.27 ms right after idle, 0.30 ms a few
+milliseconds later and 0.24-0.25 ms from about 30 ms on. A model runs for
+seconds, so the steady state is the figure of interest: before the W warmup
+steps the bench runs the same step, untimed, until --settle-ms of wall time
+have passed (`settle_steps` in the output), and every other timed loop is
+preceded by the same kind of load. --settle-ms 0 switches it off.
 """
 import argparse
 import ctypes as C
@@ -34,7 +44,7 @@ PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 matrix peak (vendor figure)
 PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E peak
 # HBM bytes one C2 attention launch moves, from the FETCH_SIZE and WRITE_SIZE hardware counters scaled by a
 # 1 GiB copy kernel (profiles/k_fa_fwd_hd128__c2__hbm_traffic.txt): 103.9 MB read + 28.3 MB written.
-C2_ATTENTION_HBM_TRAFFIC = 132_174_000
+C2_ATTENTION_HBM_TRAFFIC = 132_261_000
 
 _vp = C.c_void_p
 
@@ -169,6 +179,17 @@ class Resident:
             self.lib.iris_dev_free(p)
 
 
+def settle(lib, fn, ms):
+    """Runs fn(i) back to back, untimed, until `ms` of wall time have passed; returns the number of calls."""
+    n, t0 = 0, time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(10):
+            fn(n)
+            n += 1
+        lib.iris_dev_sync()
+    return n
+
+
 def event_time(hip, stream, fn, reps, start=0):
     """Average ms of `fn(i)` over `reps` back-to-back launches between two events."""
     a, b = hip.event(), hip.event()
@@ -179,16 +200,19 @@ def event_time(hip, stream, fn, reps, start=0):
     return hip.elapsed_ms(a, b) / reps
 
 
-def per_launch_times(hip, stream, fn, reps):
-    """Per-launch ms with an event pair around every launch (for kernels >> event cost)."""
+def per_launch_times(hip, stream, fn, reps, before=None):
+    """Per-launch ms with an event pair around every launch (for kernels >> event cost); `before(i)`, if given,
+    is enqueued ahead of each timed launch, outside its event pair."""
     evs = [(hip.event(), hip.event()) for _ in range(reps)]
     for i, (a, b) in enumerate(evs):
+        if before:
+            before(i)
         hip.record(a, stream); fn(i); hip.record(b, stream)
     return [hip.elapsed_ms(a, b) for a, b in evs]
 
 
 # ----------------------------------------------------------------------------- the other operators
-def other_ops(dev, hip, stream, rng):
+def other_ops(dev, hip, stream, rng, settle_ms=0.0):
     """Latency of the other device operators at the shapes a transformer block of the bench configuration
     uses (4608 tokens, width 3072): linear layers in TFLOP/s, one-pass kernels in GB/s (bytes read + written)."""
     lib = dev.lib
@@ -197,6 +221,7 @@ def other_ops(dev, hip, stream, rng):
 
     def timed(fn, reps=10):
         fn(0); lib.iris_dev_sync(); dev.check()
+        settle(lib, fn, settle_ms)
         return min(event_time(hip, stream, fn, reps) for _ in range(3))
 
     x = dev.to_device(to_bf16(rng.standard_normal((rows, 12288), dtype=np.float32)))
@@ -361,8 +386,11 @@ def cpu_baseline(c):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="untimed steps before the warmup until this much wall time has passed "
+                         "(the clocks need tens of ms of load to settle); 0 = none")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-configuration table")
     ap.add_argument("--no-machine", action="store_true", help="skip the MFMA-only / stream-copy ceilings")
@@ -388,6 +416,7 @@ def main():
     res = Resident(dev, c2, copies)
     flops = attention_flops(c2)
 
+    settle_steps = settle(lib, res.step, args.settle_ms)
     for i in range(args.warmup):
         res.step(i)
     lib.iris_dev_sync()
@@ -406,8 +435,10 @@ def main():
     lib.iris_dev_sync()
     fused_ms = (time.perf_counter() - t0) / args.steps * 1e3
 
-    # dominant kernel alone: events around every attention launch
-    att = per_launch_times(hip, stream, res.attention, max(args.steps, 10))
+    # dominant kernel in its place in the step: events around the attention launch of every step (Q and K rows
+    # just rewritten by the two norm calls, V rows not touched since the buffer's last turn)
+    att = per_launch_times(hip, stream, res.attention, max(args.steps, 10),
+                           before=lambda i: (res.norm_q(i), res.norm_k(i)))
     att_ms = float(np.mean(att))
     # bandwidth-bound kernel: back-to-back launches over rotating buffers (cold) and one buffer (warm)
     reps = max(args.steps, 2 * copies)
@@ -420,7 +451,8 @@ def main():
 
     out = {
         "metric": "joint_attention_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_steps": settle_steps,
+        "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "C2: norm+rope(Q), norm+rope(K), joint attention; 24 heads x 128, 512 text + 4096 image "
                                "tokens, fused qkv rows (ldi 9216), one sequence",
@@ -450,6 +482,7 @@ def main():
             r = Resident(dev, c, 2)
             for i in range(3):
                 r.step(i)
+            settle(lib, r.attention, args.settle_ms / 2)
             n = 20
             a_ms = float(np.mean(per_launch_times(hip, stream, r.attention, n)))
             qk_ms = event_time(hip, stream, r.norm_qk, n)
@@ -464,7 +497,7 @@ def main():
         out["shapes"] = shapes
 
     if not args.no_shapes:
-        out["other_ops"] = other_ops(dev, hip, stream, rng)
+        out["other_ops"] = other_ops(dev, hip, stream, rng, args.settle_ms / 5)
         out["rope_tables"] = rope_table_times(dev, c2)
     if not args.no_machine:
         out["machine"] = machine_ceilings(dev, hip, stream)
