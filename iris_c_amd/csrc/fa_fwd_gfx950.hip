@@ -565,19 +565,25 @@ extern "C" int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uin
                                  int seq_k, int heads, int kv_heads, float scale, int causal,
                                  const int *key_mask) {
     hipStream_t st = (hipStream_t)stream;
-    /* 256 queries per workgroup halve the K/V traffic from L2 per query, but one such workgroup
-     * fills a CU, so the grid runs in rounds of 256 and a badly filled last round is expensive:
-     * they are used when the rounds are at least 80 % full. 128 queries (two workgroups per CU)
-     * otherwise. A workgroup walks its key tiles one after the other, about 2 us each, so a short
-     * sequence is bound by that latency and wants many small workgroups: 64 or 32 queries when
-     * the larger shapes would leave CUs without work (measured on 24 heads, 256 .. 4608 tokens). */
+    /* A workgroup walks its key tiles one after the other, about 2 us each, so a short sequence is
+     * bound by that latency and wants many small workgroups: 32 or 64 queries when the larger
+     * shapes would leave CUs without work. From 576 waves of 32 queries on, the choice is between
+     * 256 queries (8 waves, one workgroup fills a CU, half the K/V traffic from L2 per query) and
+     * 128 queries (4 waves, two workgroups per CU), by the cost of their rounds over the 256 CUs,
+     * in units of one full round of 256-query workgroups: such a round costs 1 however few CUs it
+     * uses; a round of 128-query workgroups costs 1.13 when some CU gets two of them and 0.72 when
+     * none does (one wave per SIMD runs faster than two, not twice as fast). Constants measured on
+     * 24 heads, 256 .. 12800 tokens, clocks settled. */
     const long units = (long)((seq_q + 31) / 32) * heads;          /* waves of 32 queries */
-    const long wg256 = (long)((seq_q + 255) / 256) * heads;
-    const long rounds = (wg256 + CUS - 1) / CUS;
-    if (units >= 576 && 5 * wg256 >= 4 * rounds * CUS)
-        return launch_w<8>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
-    if (units >= 576)
+    if (units >= 576) {
+        const long wg256 = (long)((seq_q + 255) / 256) * heads, wg128 = (long)((seq_q + 127) / 128) * heads;
+        const long cost8 = 100 * ((wg256 + CUS - 1) / CUS);
+        const long rest4 = wg128 % (2 * CUS);
+        const long cost4 = 113 * (wg128 / (2 * CUS)) + (rest4 == 0 ? 0 : rest4 <= CUS ? 72 : 113);
+        if (cost8 <= cost4)
+            return launch_w<8>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
         return launch_w<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
+    }
     if (units >= 256)
         return launch_w<2>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
     return launch_w<1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
