@@ -38,7 +38,7 @@ oracle/libiris_oracle.so:
 iris_c_amd/libiris_microbench.so: $(CSRC)/microbench.hip
 	$(HIPCC) $(HIPFLAGS) -shared -o $@ $<
 
-$(CSRC)/%.o: $(CSRC)/%.hip $(CSRC)/iris_kernels_hip.h
+$(CSRC)/%.o: $(CSRC)/%.hip $(CSRC)/iris_kernels_hip.h $(CSRC)/norm_rope_math.h
 	$(HIPCC) $(HIPFLAGS) -c $< -o $@
 
 HOST_HDRS = include/iris_dev.h include/iris_rope.h $(CSRC)/iris_kernels_hip.h $(CSRC)/iris_rope_internal.h

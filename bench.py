@@ -174,6 +174,18 @@ class Resident:
         """The same work with the library's one-launch Q+K normalisation (an addition to the reference API)."""
         self.norm_qk(i); self.attention(i)
 
+    def attention_qnorm(self, i):
+        c = self.c
+        self.lib.iris_dev_attention_qnorm(self.out, c["ldo"], self.col(i, 0), self.col(i, c["q_dim"]),
+                                          self.col(i, c["q_dim"] + c["kv_dim"]), c["ldi"], c["seq"], c["seq"], c["heads"],
+                                          c["kv_heads"], c["hd"], c["scale"], int(c["causal"]), self.mask, self.wq,
+                                          self.cos, self.sin, c["eps"], c["split_half"])
+
+    def step_q_norm_in_attention(self, i):
+        """The same work with Q normalised while the attention kernel loads it (an addition to the reference API):
+        one norm launch on K, one attention launch."""
+        self.norm_k(i); self.attention_qnorm(i)
+
     def free(self):
         for p in self.bufs + [self.out, self.wq, self.wk, self.cos, self.sin] + ([self.mask] if self.mask else []):
             self.lib.iris_dev_free(p)
@@ -435,6 +447,12 @@ def main():
     lib.iris_dev_sync()
     fused_ms = (time.perf_counter() - t0) / args.steps * 1e3
 
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        res.step_q_norm_in_attention(i)
+    lib.iris_dev_sync()
+    qnorm_ms = (time.perf_counter() - t0) / args.steps * 1e3
+
     # dominant kernel in its place in the step: events around the attention launch of every step (Q and K rows
     # just rewritten by the two norm calls, V rows not touched since the buffer's last turn)
     att = per_launch_times(hip, stream, res.attention, max(args.steps, 10),
@@ -459,6 +477,8 @@ def main():
                    "device": dev.name()},
         "step_with_fused_qk_norm": {"ms_per_step": round(fused_ms, 4), "tflops": round(flops / (fused_ms * 1e-3) / 1e12, 2),
                                     "note": "two launches: iris_dev_head_norm_rope_qk + iris_dev_attention"},
+        "step_with_q_norm_in_attention": {"ms_per_step": round(qnorm_ms, 4), "tflops": round(flops / (qnorm_ms * 1e-3) / 1e12, 2),
+                                          "note": "two launches: iris_dev_head_norm_rope on K + iris_dev_attention_qnorm"},
         "roofline": {"kernel": "k_fa_fwd_hd128", "bound": "mfma", "achieved": round(flops / (att_ms * 1e-3) / 1e12, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / (att_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
                      "traffic": C2_ATTENTION_HBM_TRAFFIC, "traffic_unit": "bytes per launch (hardware counters, profiled separately)",

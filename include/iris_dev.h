@@ -134,6 +134,23 @@ void iris_dev_head_norm_rope_qk(uint16_t *xq, uint16_t *xk, int ld,
                                 int seq, int q_heads, int k_heads, int head_dim,
                                 float eps, int split_half);
 
+/* iris_dev_attention with the Q half of the normalisation folded in: the result is what
+ *     iris_dev_head_norm_rope(q, ldi, wq, rope_cos, rope_sin, seq_q, heads, head_dim, eps, split_half);
+ *     iris_dev_attention(out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, head_dim, scale, causal, key_mask);
+ * gives, bit for bit, but q is only read: the rows in memory stay as they were, and the pass
+ * that reads and rewrites them is saved. k must already be normalised (the single
+ * iris_dev_head_norm_rope call on K stays). For the call sites that use Q for nothing else
+ * after the attention, which is all of them (iris_transformer_flux.c:3834-3839,
+ * iris_transformer_flux3.c:693-696, iris_transformer_zimage.c:1948-1951, iris_qwen3.c:1590-1596).
+ * Row s of the tables belongs to query row s. Every argument combination is answered: those the
+ * matrix-core kernel does not take go through a normalised copy of Q in private scratch. */
+void iris_dev_attention_qnorm(uint16_t *out, int ldo,
+                              const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                              int ldi, int seq_q, int seq_k, int heads, int kv_heads,
+                              int head_dim, float scale, int causal, const int *key_mask,
+                              const float *wq, const float *rope_cos, const float *rope_sin,
+                              float eps, int split_half);
+
 /* The library's stream as a hipStream_t, for callers that time kernels with
  * HIP events or order their own work after the library's. */
 void *iris_dev_stream(void);

@@ -29,6 +29,8 @@ ABI = {
     "iris_dev_sync": (None, []),
     "iris_dev_head_norm_rope": (None, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _i]),
     "iris_dev_attention": (None, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp]),
+    "iris_dev_attention_qnorm": (None, [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp,
+                                        _vp, _vp, _vp, _f, _i]),
     "iris_dev_f32_to_bf16": (None, [_vp, _vp, _sz]),
     "iris_dev_linear_f32": (None, [_vp, _vp, _vp, _i, _i, _i]),
     "iris_dev_linear_bf16": (None, [_vp, _vp, _vp, _i, _i, _i]),

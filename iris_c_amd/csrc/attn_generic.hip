@@ -45,7 +45,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 __global__ void __launch_bounds__(64)
 k_attention_generic(uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k, const uint16_t *v,
-                    int ldi, int seq_q, int seq_k, int kv_group, int hd, int kstride, float scale,
+                    int ldq, int ldi, int seq_q, int seq_k, int kv_group, int hd, int kstride, float scale,
                     int causal, const int *key_mask) {
     extern __shared__ __align__(16) unsigned char smem[];
     float *qs = reinterpret_cast<float *>(smem);                 /* [QB][hd] */
@@ -59,7 +59,7 @@ k_attention_generic(uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k
 
     for (int idx = lane; idx < QB * hd; idx += 64) {
         int qq = idx / hd, d = idx - qq * hd;
-        qs[idx] = qq < nq ? bf2f(q[(size_t)(q0 + qq) * ldi + (size_t)head * hd + d]) : 0.0f;
+        qs[idx] = qq < nq ? bf2f(q[(size_t)(q0 + qq) * ldq + (size_t)head * hd + d]) : 0.0f;
     }
 
     float acc[QB][DSLOTS];
@@ -132,7 +132,7 @@ k_attention_generic(uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k
 
 }  // namespace
 
-extern "C" int iris_hip_attention_generic(void *stream, uint16_t *out, int ldo, const uint16_t *q,
+extern "C" int iris_hip_attention_generic(void *stream, uint16_t *out, int ldo, const uint16_t *q, int ldq,
                                           const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
                                           int seq_k, int heads, int kv_heads, int head_dim,
                                           float scale, int causal, const int *key_mask) {
@@ -151,6 +151,6 @@ extern "C" int iris_hip_attention_generic(void *stream, uint16_t *out, int ldo, 
     }
     dim3 grid((seq_q + QB - 1) / QB, heads);
     hipLaunchKernelGGL(k_attention_generic, grid, dim3(64), smem, (hipStream_t)stream, out, ldo, q, k, v,
-                       ldi, seq_q, seq_k, heads / kv_heads, head_dim, kstride, scale, causal, key_mask);
+                       ldq, ldi, seq_q, seq_k, heads / kv_heads, head_dim, kstride, scale, causal, key_mask);
     return (int)hipGetLastError();
 }

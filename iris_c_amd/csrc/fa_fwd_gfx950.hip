@@ -71,6 +71,12 @@
  * exponentials are taken against the older max. Softmax is invariant to that
  * shift, and exp2 arguments stay <= 8, far from overflow.
  *
+ * Optionally (iris_dev_attention_qnorm, no counterpart in the reference) the per-head RMSNorm
+ * and rotary embedding of Q (reference iris_cuda.cu:402-420) are applied to the Q fragments
+ * right after they are loaded, with the operations of the stand-alone kernel in the same
+ * order, so that the result equals norm-then-attention bit for bit and the separate pass
+ * over Q is saved. It is a run-time branch of the prologue, not another instantiation.
+ *
  * Workgroups are numbered so that each XCD (own L2) walks a contiguous range
  * of (head, query-tile) pairs: the K/V of a head are then fetched into one
  * L2 instead of eight.
@@ -79,6 +85,7 @@
 #include <stdint.h>
 
 #include "iris_kernels_hip.h"
+#include "norm_rope_math.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -215,12 +222,93 @@ __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+/* Optional RMSNorm + rotary embedding of Q while it is loaded (w == nullptr: Q is taken as it
+ * is). cos/sin rows belong to the query rows, as in iris_dev_head_norm_rope. */
+struct QNorm {
+    const float *w, *rope_cos, *rope_sin;
+    float eps;
+    int split_half;
+};
+
+/* Sum over the four lanes l%16, +16, +32, +48, paired (l, l+32) first and then (l, l+16): with
+ * the lane in 16-lane row g holding u[g] this is (u[0] + u[2]) + (u[1] + u[3]). */
+__device__ __forceinline__ float quad_group_sum_02_13(float v) {
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    const float w = __uint_as_float(b[0]) + __uint_as_float(b[1]);
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(w), __float_as_uint(w), false, false);
+    return __uint_as_float(a[0]) + __uint_as_float(a[1]);
+}
+
+/* Normalises and rotates the 32 dims of one query that a lane holds as B operands: chunk
+ * c = 4 ks + lg (dims 8c .. 8c+7) in qb[ks], the other chunks of the query in the lanes 16, 32
+ * and 48 away. Same operations in the same order as k_norm_rope_hd128 (norm_rope_math.h), so the
+ * operand bits equal what that kernel would have stored. */
+__device__ __forceinline__ void norm_rope_q_fragment(bf16x8 (&qb)[4], const QNorm &qn, int row, int lg) {
+    float e[4][8], p[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+        const u32x4 raw = __builtin_bit_cast(u32x4, qb[ks]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            e[ks][2 * j] = __uint_as_float(raw[j] << 16);
+            e[ks][2 * j + 1] = __uint_as_float(raw[j] & 0xffff0000u);
+        }
+        p[ks] = nr_chunk_sum_squares(e[ks]);
+    }
+    /* chunks lg, lg+4, lg+8, lg+12: t[lg] = p0 + p2, t[lg+4] = p1 + p3, u[lg] = t[lg] + t[lg+4] */
+    const float inv = nr_inv_rms128(quad_group_sum_02_13((p[0] + p[2]) + (p[1] + p[3])), qn.eps);
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+        const float4 w0 = *reinterpret_cast<const float4 *>(qn.w + 32 * ks + 8 * lg);
+        const float4 w1 = *reinterpret_cast<const float4 *>(qn.w + 32 * ks + 8 * lg + 4);
+        const float w8[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) e[ks][i] = nr_scaled(e[ks][i], inv, w8[i]);
+    }
+    const float *ct = qn.rope_cos + (size_t)row * 64, *st = qn.rope_sin + (size_t)row * 64;
+    float o[4][8];
+    if (qn.split_half) {
+        /* pairs (d, d + 64): chunk c < 8 holds a, chunk c + 8 (k-step ks + 2 of the same lane) holds b;
+         * table columns 8c .. 8c+7 */
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            const int col = 32 * ks + 8 * lg;
+            const float4 c0 = *reinterpret_cast<const float4 *>(ct + col), c1 = *reinterpret_cast<const float4 *>(ct + col + 4);
+            const float4 s0 = *reinterpret_cast<const float4 *>(st + col), s1 = *reinterpret_cast<const float4 *>(st + col + 4);
+            const float cv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+            const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                o[ks][i] = nr_rot_first(e[ks][i], e[ks + 2][i], cv[i], sv[i]);
+                o[ks + 2][i] = nr_rot_second(e[ks][i], e[ks + 2][i], cv[i], sv[i]);
+            }
+        }
+    } else {
+        /* pairs (2i, 2i+1): four per chunk, table columns 4c .. 4c+3 */
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            const int col = 16 * ks + 4 * lg;
+            const float4 c4 = *reinterpret_cast<const float4 *>(ct + col), s4 = *reinterpret_cast<const float4 *>(st + col);
+            const float cv[4] = {c4.x, c4.y, c4.z, c4.w}, sv[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                o[ks][2 * j] = nr_rot_first(e[ks][2 * j], e[ks][2 * j + 1], cv[j], sv[j]);
+                o[ks][2 * j + 1] = nr_rot_second(e[ks][2 * j], e[ks][2 * j + 1], cv[j], sv[j]);
+            }
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++)
+        qb[ks] = __builtin_bit_cast(bf16x8, u32x4{pack_bf16(o[ks][0], o[ks][1]), pack_bf16(o[ks][2], o[ks][3]),
+                                                  pack_bf16(o[ks][4], o[ks][5]), pack_bf16(o[ks][6], o[ks][7])});
+}
+
 template <int WAVES, bool CAUSAL, bool MASK>
 __global__ void __launch_bounds__(64 * WAVES, 2)
 k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ q,
                const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
                int seq_q, int seq_k, int q_tiles, int total_work, int work_per_xcd,
-               int kv_group, float scale_log2, const int *__restrict__ key_mask) {
+               int kv_group, float scale_log2, const int *__restrict__ key_mask, QNorm qnorm) {
     extern __shared__ __align__(16) uint16_t lds[];     /* NSTAGE stages of [K tile | V tile] */
     constexpr int BM = 32 * WAVES, NI = 32 / WAVES;
     /* Key tiles between two barriers. Two for the 8-wave shape (one workgroup per CU, so the LDS
@@ -246,17 +334,6 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 
     const uint16_t *kbase = k + (size_t)kvh * HD;
     const uint16_t *vbase = v + (size_t)kvh * HD;
-
-    /* Q^T as B operands: for query block nb and k-step ks the lane holds dims 32ks + 8lg .. +7
-     * of query 16nb + li. */
-    bf16x8 qb[2][4];
-#pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
-        const uint16_t *qp = q + (size_t)min(qrow0 + 16 * nb, seq_q - 1) * ldi + (size_t)head * HD + 8 * lg;
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++)
-            qb[nb][ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 32 * ks));
-    }
 
     f32x4 o[8][2];                                   /* O^T: dims 16db + 4lg + r of query block nb */
 #pragma unroll
@@ -313,11 +390,31 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         }
     }
 
-    /* The tile requests below are invisible to the compiler's own wait-count bookkeeping, so every
-     * load it does know about (Q) is completed here: the empty asm consumes the registers, which
-     * pins the loads and their wait before this point. Left to itself the compiler sinks the Q
-     * loads to the loop and re-waits for them in every iteration, which in fact waits for the
-     * newest tile requests. */
+    /* ---- prologue: the first group of tiles is requested before Q, so that the two fetches overlap ---- */
+#pragma unroll
+    for (int t = 0; t < GROUP; t++) request(t, t);
+
+    /* Q^T as B operands: for query block nb and k-step ks the lane holds dims 32ks + 8lg .. +7
+     * of query 16nb + li. */
+    bf16x8 qb[2][4];
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+        const uint16_t *qp = q + (size_t)min(qrow0 + 16 * nb, seq_q - 1) * ldi + (size_t)head * HD + 8 * lg;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+            qb[nb][ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 32 * ks));
+    }
+    if (qnorm.w) {                                   /* wave-uniform */
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) norm_rope_q_fragment(qb[nb], qnorm, min(qrow0 + 16 * nb, seq_q - 1), lg);
+    }
+
+    /* The tile requests are invisible to the compiler's own wait-count bookkeeping, so every load it
+     * does know about (Q, the norm weights and tables) is completed here: the empty asm consumes the
+     * registers, which pins the loads and their wait before this point. (Waiting for them also waits
+     * for the older tile requests above, which the barrier below needs anyway.) Left to itself the
+     * compiler sinks the Q loads to the loop and re-waits for them in every iteration, which in fact
+     * waits for the newest tile requests. */
 #pragma unroll
     for (int nb = 0; nb < 2; nb++)
 #pragma unroll
@@ -327,9 +424,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             qb[nb][ks] = __builtin_bit_cast(bf16x8, t);
         }
 
-    /* ---- prologue: the first group of tiles landed ---- */
-#pragma unroll
-    for (int t = 0; t < GROUP; t++) request(t, t);
+    /* the first group of tiles has landed */
     wait_vmcnt<0>();
     lds_barrier();                                       /* also publishes the key-mask words */
 
@@ -526,7 +621,7 @@ constexpr int CUS = 256;
 template <int W, bool C, bool M>
 int launch(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
            const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads,
-           float scale, const int *key_mask) {
+           float scale, const int *key_mask, const QNorm &qn) {
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd128<W, C, M>),
@@ -542,29 +637,27 @@ int launch(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint
     if (lds_bytes > LDS_MAX) return (int)hipErrorInvalidValue;       /* the caller keeps masked seq_k below the limit */
     hipLaunchKernelGGL((k_fa_fwd_hd128<W, C, M>), dim3(per_xcd * XCDS), dim3(64 * W), lds_bytes, st, out, ldo,
                        q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, heads / kv_heads,
-                       scale * 1.4426950408889634f, key_mask);
+                       scale * 1.4426950408889634f, key_mask, qn);
     return (int)hipGetLastError();
 }
 
 template <int W>
 int launch_w(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
              const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads, float scale,
-             int causal, const int *key_mask) {
+             int causal, const int *key_mask, const QNorm &qn) {
     if (causal) {
-        if (key_mask) return launch<W, true, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask);
-        return launch<W, true, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask);
+        if (key_mask) return launch<W, true, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
+        return launch<W, true, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
     }
-    if (key_mask) return launch<W, false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask);
-    return launch<W, false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask);
+    if (key_mask) return launch<W, false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
+    return launch<W, false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
 }
 
 }  // namespace
 
-extern "C" int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uint16_t *q,
-                                 const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
-                                 int seq_k, int heads, int kv_heads, float scale, int causal,
-                                 const int *key_mask) {
-    hipStream_t st = (hipStream_t)stream;
+static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
+                            const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads, float scale,
+                            int causal, const int *key_mask, const QNorm &qn) {
     /* A workgroup walks its key tiles one after the other, about 2 us each, so a short sequence is
      * bound by that latency and wants many small workgroups: 32 or 64 queries when the larger
      * shapes would leave CUs without work. From 576 waves of 32 queries on, the choice is between
@@ -581,10 +674,31 @@ extern "C" int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uin
         const long rest4 = wg128 % (2 * CUS);
         const long cost4 = 113 * (wg128 / (2 * CUS)) + (rest4 == 0 ? 0 : rest4 <= CUS ? 72 : 113);
         if (cost8 <= cost4)
-            return launch_w<8>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
-        return launch_w<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
+            return launch_w<8>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+        return launch_w<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
     }
     if (units >= 256)
-        return launch_w<2>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
-    return launch_w<1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask);
+        return launch_w<2>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+    return launch_w<1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+}
+
+extern "C" int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uint16_t *q,
+                                 const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
+                                 int seq_k, int heads, int kv_heads, float scale, int causal,
+                                 const int *key_mask) {
+    const QNorm none = {nullptr, nullptr, nullptr, 0.0f, 0};
+    return launch_any_width((hipStream_t)stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal,
+                            key_mask, none);
+}
+
+/* The same with Q normalised and rotated while it is loaded (w, rope_cos, rope_sin 16-byte aligned). */
+extern "C" int iris_hip_fa_hd128_qnorm(void *stream, uint16_t *out, int ldo, const uint16_t *q,
+                                       const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
+                                       int seq_k, int heads, int kv_heads, float scale, int causal,
+                                       const int *key_mask, const float *w, const float *rope_cos,
+                                       const float *rope_sin, float eps, int split_half) {
+    if (!w || !rope_cos || !rope_sin) return (int)hipErrorInvalidValue;
+    const QNorm qn = {w, rope_cos, rope_sin, eps, split_half != 0};
+    return launch_any_width((hipStream_t)stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal,
+                            key_mask, qn);
 }

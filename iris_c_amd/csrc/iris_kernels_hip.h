@@ -36,6 +36,15 @@ int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uint16_t *q,
                       const uint16_t *k, const uint16_t *v, int ldi, int seq_q, int seq_k,
                       int heads, int kv_heads, float scale, int causal, const int *key_mask);
 
+/* The same with the per-head RMSNorm + rotary embedding of Q (weights w[128], tables
+ * [seq_q, 64], all 16-byte aligned) applied while Q is loaded; q itself is only read. The Q
+ * operand has the bits that iris_hip_norm_rope_hd128 would have stored. */
+int iris_hip_fa_hd128_qnorm(void *stream, uint16_t *out, int ldo, const uint16_t *q,
+                            const uint16_t *k, const uint16_t *v, int ldi, int seq_q, int seq_k,
+                            int heads, int kv_heads, float scale, int causal, const int *key_mask,
+                            const float *w, const float *rope_cos, const float *rope_sin, float eps,
+                            int split_half);
+
 /* head_dim 256 or 512 (the VAE's single 512-wide head): the head dim is cut into slices of
  * 128 that a group of waves shares; same argument conditions as iris_hip_fa_hd128. */
 int iris_hip_fa_sliced(void *stream, uint16_t *out, int ldo, const uint16_t *q,
@@ -43,8 +52,9 @@ int iris_hip_fa_sliced(void *stream, uint16_t *out, int ldo, const uint16_t *q,
                        int heads, int kv_heads, int head_dim, float scale, int causal,
                        const int *key_mask);
 
-/* Any head_dim <= 512, any stride / alignment / scale. Correctness path. */
-int iris_hip_attention_generic(void *stream, uint16_t *out, int ldo, const uint16_t *q,
+/* Any head_dim <= 512, any stride / alignment / scale; the rows of q may have a stride (ldq) of
+ * their own. Correctness path. */
+int iris_hip_attention_generic(void *stream, uint16_t *out, int ldo, const uint16_t *q, int ldq,
                                const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
                                int seq_k, int heads, int kv_heads, int head_dim, float scale,
                                int causal, const int *key_mask);

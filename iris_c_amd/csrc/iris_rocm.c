@@ -33,6 +33,9 @@ static const char *g_last_kernel = "none";
 static uint16_t *g_conv_scratch = NULL;
 static float *g_gn_scratch = NULL;
 static size_t g_gn_scratch_floats = 0;
+/* normalised copy of Q for the iris_dev_attention_qnorm calls that the matrix-core kernel does not take */
+static uint16_t *g_q_scratch = NULL;
+static size_t g_q_scratch_bytes = 0;
 /* positions and column frequencies of the rotary tables being generated */
 static void *g_rope_stage = NULL;
 static size_t g_rope_stage_bytes = 0;
@@ -92,6 +95,9 @@ void iris_dev_cleanup(void) {
     if (g_conv_scratch) check(hipFree(g_conv_scratch), "free");
     if (g_gn_scratch) check(hipFree(g_gn_scratch), "free");
     if (g_rope_stage) check(hipFree(g_rope_stage), "free");
+    if (g_q_scratch) check(hipFree(g_q_scratch), "free");
+    g_q_scratch = NULL;
+    g_q_scratch_bytes = 0;
     iris_lt_release();
     g_conv_scratch = NULL;
     g_gn_scratch = NULL;
@@ -191,33 +197,93 @@ void iris_dev_head_norm_rope_qk(uint16_t *xq, uint16_t *xk, int ld,
               split_half);
 }
 
-void iris_dev_attention(uint16_t *out, int ldo,
-                        const uint16_t *q, const uint16_t *k, const uint16_t *v,
-                        int ldi, int seq_q, int seq_k, int heads, int kv_heads,
-                        int head_dim, float scale, int causal, const int *key_mask) {
-    if (!need_ready("attention")) return;
+/* wq == NULL: plain attention. Otherwise Q is normalised and rotated on the way in. */
+static void attention(const char *what, uint16_t *out, int ldo,
+                      const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                      int ldi, int seq_q, int seq_k, int heads, int kv_heads,
+                      int head_dim, float scale, int causal, const int *key_mask,
+                      const float *wq, const float *rope_cos, const float *rope_sin,
+                      float eps, int split_half) {
+    if (!need_ready(what)) return;
     if (seq_q <= 0 || heads <= 0) return;
     if (kv_heads <= 0 || heads % kv_heads != 0 || head_dim <= 0 || head_dim > 512 || seq_k < 0) {
-        fail(-1, "attention", "need heads % kv_heads == 0, 0 < head_dim <= 512, seq_k >= 0");
+        fail(-1, what, "need heads % kv_heads == 0, 0 < head_dim <= 512, seq_k >= 0");
+        return;
+    }
+    if (wq && (!rope_cos || !rope_sin || (head_dim & 1))) {
+        fail(-1, what, "need the rotary tables and an even head_dim");
         return;
     }
     int mfma_ok = seq_k > 0 && scale > 0.0f && ldi % 8 == 0 && ldo % 4 == 0 &&
                   aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out, 8);
     int err;
-    if (mfma_ok && head_dim == 128 && (!key_mask || seq_k <= IRIS_FA_MAX_MASKED_KEYS)) {
-        g_last_kernel = "fa_hd128";
-        err = iris_hip_fa_hd128(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads,
-                                scale, causal != 0, key_mask);
+    if (mfma_ok && head_dim == 128 && (!key_mask || seq_k <= IRIS_FA_MAX_MASKED_KEYS) &&
+        (!wq || (aligned(wq, 16) && aligned(rope_cos, 16) && aligned(rope_sin, 16)))) {
+        if (wq) {
+            g_last_kernel = "fa_hd128_qnorm";
+            err = iris_hip_fa_hd128_qnorm(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads,
+                                          scale, causal != 0, key_mask, wq, rope_cos, rope_sin, eps, split_half != 0);
+        } else {
+            g_last_kernel = "fa_hd128";
+            err = iris_hip_fa_hd128(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads,
+                                    scale, causal != 0, key_mask);
+        }
+    } else if (wq) {
+        /* a normalised copy of Q (rows of heads * head_dim) in private scratch, then the generic kernel,
+         * which takes a row stride of its own for q */
+        const int ldq = heads * head_dim;
+        const size_t need = (size_t)seq_q * ldq * sizeof(uint16_t);
+        if (need > g_q_scratch_bytes) {
+            if (g_q_scratch) {
+                check(hipStreamSynchronize(g_stream), "sync");
+                check(hipFree(g_q_scratch), "free");
+            }
+            g_q_scratch = NULL;
+            g_q_scratch_bytes = 0;
+            if (hipMalloc((void **)&g_q_scratch, need) != hipSuccess) {
+                (void)hipGetLastError();
+                g_q_scratch = NULL;
+                fail(-1, what, "scratch allocation failed");
+                return;
+            }
+            g_q_scratch_bytes = need;
+        }
+        if (!check(hipMemcpy2DAsync(g_q_scratch, (size_t)ldq * 2, q, (size_t)ldi * 2, (size_t)ldq * 2, (size_t)seq_q,
+                                    hipMemcpyDeviceToDevice, g_stream), "copy of q"))
+            return;
+        norm_rope(g_q_scratch, NULL, ldq, wq, NULL, rope_cos, rope_sin, seq_q, heads, 0, head_dim, eps, split_half);
+        g_last_kernel = "attention_generic_qnorm";
+        err = iris_hip_attention_generic(g_stream, out, ldo, g_q_scratch, ldq, k, v, ldi, seq_q, seq_k, heads,
+                                         kv_heads, head_dim, scale, causal != 0, key_mask);
     } else if (mfma_ok && (head_dim == 256 || head_dim == 512)) {
         g_last_kernel = "fa_sliced";
         err = iris_hip_fa_sliced(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads,
                                  head_dim, scale, causal != 0, key_mask);
     } else {
         g_last_kernel = "attention_generic";
-        err = iris_hip_attention_generic(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads,
+        err = iris_hip_attention_generic(g_stream, out, ldo, q, ldi, k, v, ldi, seq_q, seq_k, heads,
                                          kv_heads, head_dim, scale, causal != 0, key_mask);
     }
     if (err) check((hipError_t)err, "attention launch");
+}
+
+void iris_dev_attention(uint16_t *out, int ldo,
+                        const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                        int ldi, int seq_q, int seq_k, int heads, int kv_heads,
+                        int head_dim, float scale, int causal, const int *key_mask) {
+    attention("attention", out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, head_dim, scale, causal, key_mask,
+              NULL, NULL, NULL, 0.0f, 0);
+}
+
+void iris_dev_attention_qnorm(uint16_t *out, int ldo,
+                              const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                              int ldi, int seq_q, int seq_k, int heads, int kv_heads,
+                              int head_dim, float scale, int causal, const int *key_mask,
+                              const float *wq, const float *rope_cos, const float *rope_sin,
+                              float eps, int split_half) {
+    if (!wq) { fail(-1, "attention_qnorm", "the norm weights are missing"); return; }
+    attention("attention_qnorm", out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, head_dim, scale, causal,
+              key_mask, wq, rope_cos, rope_sin, eps, split_half);
 }
 
 /* ---- the other operators: thin checked wrappers over the launchers ---- */

@@ -22,6 +22,7 @@
 #include <stdint.h>
 
 #include "iris_kernels_hip.h"
+#include "norm_rope_math.h"
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -119,13 +120,10 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
         if (!ptr[u]) continue;
         float e[8] = {bf_lo(raw[u].x), bf_hi(raw[u].x), bf_lo(raw[u].y), bf_hi(raw[u].y),
                       bf_lo(raw[u].z), bf_hi(raw[u].z), bf_lo(raw[u].w), bf_hi(raw[u].w)};
-        float ss = 0.0f;
+        const float ss = row16_sum(nr_chunk_sum_squares(e));
+        const float inv = nr_inv_rms128(ss, eps);
 #pragma unroll
-        for (int i = 0; i < 8; i++) ss = fmaf(e[i], e[i], ss);
-        ss = row16_sum(ss);
-        const float inv = 1.0f / sqrtf(ss * (1.0f / 128.0f) + eps);
-#pragma unroll
-        for (int i = 0; i < 8; i++) e[i] *= inv * (isk[u] ? wk8[i] : wq8[i]);
+        for (int i = 0; i < 8; i++) e[i] = nr_scaled(e[i], inv, isk[u] ? wk8[i] : wq8[i]);
 
         float o[8];
         if (SPLIT) {
@@ -134,7 +132,9 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
 #pragma unroll
             for (int i = 0; i < 8; i++) {
                 /* lanes 0-7 hold a (first half), lanes 8-15 hold b: a*c - b*s / b*c + a*s */
-                float other = row16_partner8(e[i]);
+                /* nr_rot_first(e, other) on the a lanes, nr_rot_second(other, e) on the b lanes, as one
+                 * expression: the sign flip is exact */
+                const float other = row16_partner8(e[i]);
                 o[i] = fmaf(sgn * other, sv[i], e[i] * cv[i]);
             }
         } else {
@@ -142,9 +142,9 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
             const float sv[4] = {st[u][0].x, st[u][0].y, st[u][0].z, st[u][0].w};
 #pragma unroll
             for (int p = 0; p < 4; p++) {
-                float a = e[2 * p], b = e[2 * p + 1];
-                o[2 * p] = fmaf(-b, sv[p], a * cv[p]);
-                o[2 * p + 1] = fmaf(a, sv[p], b * cv[p]);
+                const float a = e[2 * p], b = e[2 * p + 1];
+                o[2 * p] = nr_rot_first(a, b, cv[p], sv[p]);
+                o[2 * p + 1] = nr_rot_second(a, b, cv[p], sv[p]);
             }
         }
         u32x4 out;

@@ -5,7 +5,8 @@
  * (iris_transformer_flux.c:3834-3839): per-head RMSNorm + RoPE on Q, on K,
  * then joint attention, on the fused q|k|v row buffer, through the entry
  * points of include/iris_dev.h only, and compares every output element with
- * the CPU oracle run on the same inputs. The device side takes its rotary
+ * the CPU oracle run on the same inputs; the library's one-call form of the
+ * Q normalisation + attention is held to the two calls bit for bit. The device side takes its rotary
  * tables from the library's own generators (include/iris_rope.h), the oracle
  * side from the oracle's, so the table builders are part of what is checked.
  * A second pass covers the causal
@@ -76,14 +77,26 @@ static void block_case(const char *name, int seq, int heads, int kv_heads, int s
     float *d_wq = to_device(wq, sizeof wq), *d_wk = to_device(wk, sizeof wk);
     int *d_mask = mask ? to_device(mask, (size_t)seq * sizeof(int)) : NULL;
     uint16_t *d_out = iris_dev_alloc((size_t)seq * ldo * 2);
-    iris_dev_head_norm_rope(d_rows, ldi, d_wq, d_cos, d_sin, seq, heads, hd, eps, split_half);
+    uint16_t *d_out_fused = iris_dev_alloc((size_t)seq * ldo * 2);
     iris_dev_head_norm_rope(d_rows + qd, ldi, d_wk, d_cos, d_sin, seq, kv_heads, hd, eps, split_half);
+    /* the library's one-call form of "normalise Q, then attend", on the still raw Q ... */
+    iris_dev_attention_qnorm(d_out_fused, ldo, d_rows, d_rows + qd, d_rows + qd + kd, ldi, seq, seq, heads, kv_heads, hd,
+                             scale, causal, d_mask, d_wq, d_cos, d_sin, eps, split_half);
+    /* ... and the reference's two calls */
+    iris_dev_head_norm_rope(d_rows, ldi, d_wq, d_cos, d_sin, seq, heads, hd, eps, split_half);
     iris_dev_attention(d_out, ldo, d_rows, d_rows + qd, d_rows + qd + kd, ldi, seq, seq, heads, kv_heads, hd,
                        scale, causal, d_mask);
     uint16_t *rows_back = malloc((size_t)seq * ldi * 2), *out = malloc((size_t)seq * ldo * 2);
+    uint16_t *out_fused = malloc((size_t)seq * ldo * 2);
     iris_dev_download(rows_back, d_rows, (size_t)seq * ldi * 2);
     iris_dev_download(out, d_out, (size_t)seq * ldo * 2);
+    iris_dev_download(out_fused, d_out_fused, (size_t)seq * ldo * 2);
     if (iris_dev_last_error() != 0) { printf("%s: device error\n", name); failures++; }
+    {
+        const int same = memcmp(out, out_fused, (size_t)seq * ldo * 2) == 0;
+        printf("%-34s %s\n", "  attention_qnorm == the two calls", same ? "bit for bit" : "FAIL");
+        if (!same) failures++;
+    }
 
     /* oracle: same bf16 rows, same order of operations */
     orc_head_norm_rope_bf16(rows, ldi, wq, cos_t, sin_t, seq, heads, hd, eps, split_half);
@@ -102,8 +115,8 @@ static void block_case(const char *name, int seq, int heads, int kv_heads, int s
 
     iris_dev_free(d_rows); iris_dev_free(d_wq); iris_dev_free(d_wk); iris_dev_free(d_cos); iris_dev_free(d_sin);
     if (d_mask) iris_dev_free(d_mask);
-    iris_dev_free(d_out);
-    free(rows); free(rows_back); free(out); free(rows_f); free(want);
+    iris_dev_free(d_out); iris_dev_free(d_out_fused);
+    free(rows); free(rows_back); free(out); free(out_fused); free(rows_f); free(want);
 }
 
 static void vae_case(int seq, uint64_t seed) {

@@ -78,6 +78,26 @@ class Dev:
         return out, kernel
 
 
+    def attention_qnorm(self, buf, ldi, qcol, kcol, vcol, seq_q, seq_k, heads, kv_heads, hd, scale, wq, cos, sin, eps,
+                        split_half, causal=False, key_mask=None, ldo=None):
+        """iris_dev_attention_qnorm on a host buffer image. Returns (output rows as uint16 [seq_q, ldo], kernel name,
+        the buffer as it is in device memory after the call)."""
+        ldo = ldo or heads * hd
+        d = self.put(buf)
+        out0 = np.full((max(seq_q, 1), ldo), 0x7fc0, dtype=np.uint16)
+        do = self.put(out0)
+        dm = self.put(np.ascontiguousarray(key_mask, dtype=np.int32)) if key_mask is not None else None
+        dw, dc, ds = self.put(wq.astype(np.float32)), self.put(cos.astype(np.float32)), self.put(sin.astype(np.float32))
+        self.lib.iris_dev_attention_qnorm(do, ldo, ptr_add(d, 2 * qcol), ptr_add(d, 2 * kcol), ptr_add(d, 2 * vcol), ldi,
+                                          seq_q, seq_k, heads, kv_heads, hd, scale, int(causal), dm, dw, dc, ds, eps,
+                                          int(split_half))
+        self.check()
+        kernel = self.dev.last_kernel()
+        out, after = self.get(do, out0.shape, np.uint16), self.get(d, buf.shape, np.uint16)
+        self.free_all()
+        return out, kernel, after
+
+
 def error_stats(got, want):
     diff = np.abs(got.astype(np.float64) - want.astype(np.float64))
     return float(diff.max()), float(diff.mean())
