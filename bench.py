@@ -342,10 +342,19 @@ def machine_ceilings(dev, hip, stream):
     mb.iris_mb_copy(stream, b, a, n)
     cp = min(event_time(hip, stream, lambda i: mb.iris_mb_copy(stream, b, a, n), 2) for _ in range(3))
     rw = min(event_time(hip, stream, lambda i: mb.iris_mb_rmw(stream, a, n), 2) for _ in range(3))
+    # the same in-place update at the size of ONE norm+rope call of the bench workload (27 MiB of rows), on 24
+    # rotating buffers so that the rows come from HBM: what a launch of that size can reach at all
+    small = 27 << 20
+    ring = [lib.iris_dev_alloc(small) for _ in range(24)]
+    assert all(ring)
+    settle(lib, lambda i: mb.iris_mb_rmw(stream, _vp(ring[i % 24]), small), 20)
+    rw_small = min(event_time(hip, stream, lambda i: mb.iris_mb_rmw(stream, _vp(ring[i % 24]), small), 48) for _ in range(3))
     dev.check()
-    for p in (sink, a, b, ops):
+    for p in [sink, a, b, ops] + ring:
         lib.iris_dev_free(p)
-    return {"mfma_only_tflops": round(mfma, 1), "mfma_only_frac_of_peak": round(mfma / PEAK_BF16_TFLOPS, 4),
+    return {"inplace_update_27mib_cold_us": round(rw_small * 1e3, 2),
+            "inplace_update_27mib_cold_gbps": round(2 * small / rw_small / 1e6, 1),
+            "mfma_only_tflops": round(mfma, 1), "mfma_only_frac_of_peak": round(mfma / PEAK_BF16_TFLOPS, 4),
             "mfma_only_normal_data_tflops": round(mfma_data, 1),
             "mfma_only_normal_data_frac_of_peak": round(mfma_data / PEAK_BF16_TFLOPS, 4),
             "mfma16x16x32_only_normal_data_tflops": round(mfma_data16, 1),
@@ -354,7 +363,8 @@ def machine_ceilings(dev, hip, stream):
             "note": "measured ceilings of this GPU: a pure 32x32x16 MFMA loop on constant operands (short burst), "
                     "the same and the 16x16x32 shape (the one the attention kernel uses) on N(0,1) operands "
                     "(sustained; the clock drops with the data-dependent power draw), and "
-                    "streaming 16 B per lane, bytes counted read + written"}
+                    "streaming 16 B per lane, bytes counted read + written; inplace_update_27mib_cold is the "
+                    "plain update at the data volume of one norm+rope call (launch gaps included, like norm_rope.*)"}
 
 
 # ----------------------------------------------------------------------------- CPU baseline
