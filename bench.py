@@ -395,7 +395,24 @@ def cpu_baseline(c):
     t2 = time.perf_counter()
     oracle.oracle().flux2_joint_tables(*c["layout"])     # the reference's routine restated: libm on every entry
     dtab = time.perf_counter() - t2
+    # the reference's own CPU attention (its generic, BLAS-free build, compiled from its sources where they were
+    # present), when that library travelled with the tree: 6 of the heads, one thread
+    ref_leg = None
+    ref = oracle.reference()
+    if ref is not None and not c["causal"] and c["key_mask"] is None and c["heads"] == c["kv_heads"]:
+        nh = min(6, c["heads"])
+        qs, ks, vs = (np.ascontiguousarray(a[:, :nh * c["hd"]]) for a in (q, k, v))
+        o = np.empty_like(qs)
+        ptr = lambda a: a.ctypes.data_as(_vp)
+        t3 = time.perf_counter()
+        ref.lib.iris_flash_attention(ptr(o), ptr(qs), ptr(ks), ptr(vs), C.c_int(c["seq"]), C.c_int(c["seq"]), C.c_int(nh),
+                                     C.c_int(c["hd"]), C.c_float(c["scale"]))
+        dr = time.perf_counter() - t3
+        ref_leg = {"value": round(flops * nh / c["heads"] / dr / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "kind": "reference",
+                   "sample": f"iris_flash_attention of the compiled reference (its generic BLAS-free build, -O3 -ffast-math -mavx2 -mfma) on "
+                             f"{nh} of the {c['heads']} heads, all {c['seq']} tokens: {dr:.2f} s"}
     return {"value": round(flops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "reference_generic_build": ref_leg,
             "sample": f"{calls} full {c['name']} attention calls ({c['heads']}h x {c['seq']} tok, f32), mean of the last "
                       f"{calls - 1}: {dt:.2f} s each; "
                       f"sgemm from {os.path.basename(base.provider)}; host has {cores} CPUs online",
