@@ -11,6 +11,9 @@
  * the 16x16 accumulator a lane then holds four consecutive n of one output row m,
  * a single 16-byte (f32) or 8-byte (bf16) store.
  *
+ * Two kernels. Shapes with M, N >= 256 and K a multiple of 64 (every linear layer of the models at
+ * their sequence lengths) take k_gemm_dma: 256 x 256 tiles, 8 waves, tiles loaded straight into
+ * LDS, described where it is defined. Everything else with K a multiple of 8 takes k_gemm_bf16:
  * Workgroup = WM x WN waves (2 x 2 in use), tile 128 (m) x 128 (n), K in steps of 64; a wave owns
  * 64 x 64 = 4 x 4 accumulator blocks and reads 8 operands from LDS per 16 MFMAs. One
  * LDS stage of [W tile | x tile], rows padded to 160 B so that the 16 lanes the LDS
@@ -148,6 +151,198 @@ k_gemm_bf16(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t 
     }
 }
 
+/* ---- the large-shape kernel: 256 x 256 tiles, 8 waves, tiles straight from HBM/L2 into LDS ----
+ *
+ * For M, N >= 256 and K a multiple of 64. A workgroup is 8 waves (two per SIMD, one workgroup per
+ * CU), 2 along m x 4 along n, each wave owning 128 (m) x 64 (n) outputs = 8 x 4 accumulator
+ * blocks: 12 operand reads from LDS feed 32 MFMAs per k-step. K advances in tiles of 64; a stage
+ * holds the W tile (256 rows of 128 B) and the x tile (256 rows), 64 KB, two stages. The tiles
+ * are written by global_load_lds_dwordx4 (64 lanes x 16 B = eight 128 B rows per instruction,
+ * no registers, no LDS-write instructions), 8 such loads per wave and k tile (waves 0-3 the W
+ * rows, 4-7 the x rows), requested one k tile ahead; one barrier per k tile.
+ *
+ * Direct loads cannot pad rows, so the 16 B chunk c of tile row r is kept in slot
+ * c ^ ((r >> 1) & 7) of its row, the permutation applied to the source address of the lane that
+ * fills the slot. A 128-bit LDS read serves 16 lanes per pass: 16 different rows, eight of them
+ * with chunk c0 and eight with c0 + 1, and of each parity of row four with either. Two
+ * consecutive rows span the 64 banks once, so rows of equal parity must differ in slot: the
+ * rows with chunk c0 have (r >> 1) & 7 in {0, 1, 6, 7} (or {2, 3, 4, 5}), those with c0 + 1 the
+ * complement, and c0 is a multiple of 2, which makes the eight slots distinct. */
+constexpr int DT = 256;                          /* tile edge (m and n) */
+constexpr int DSTAGE = 2 * DT * TK;              /* elements per stage: W tile then x tile */
+
+__device__ __forceinline__ uint32_t lds_address(const uint16_t *p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+
+template <typename OUT>
+__global__ void __launch_bounds__(512, 2)
+k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *__restrict__ W,
+           int M, int N, int K, int tiles_m, int total, int per_xcd) {
+    extern __shared__ __align__(16) uint16_t dlds[];          /* two stages */
+    /* each XCD (own L2) walks a contiguous range of the tile list, m fastest: neighbours share a W tile */
+    const int work = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (work >= total) return;
+    const int bm = work % tiles_m, bn = work / tiles_m;
+    const int m0 = bm * DT, n0 = bn * DT;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+    const int wm = wave & 1, wn = wave >> 1;
+
+    /* this wave's share of a stage: rows 64 (wave % 4) .. +63 of the W tile (waves 0-3) or the x tile */
+    const bool loads_w = wave < 4;
+    const int row0 = 64 * (wave & 3);                          /* first row of the share inside its tile */
+    const int rows_left = (loads_w ? N - n0 : M - m0) - row0;  /* rows of the share that exist (may be <= 0) */
+    const uint16_t *share = (loads_w ? W + (size_t)n0 * K : x + (size_t)m0 * K) + (size_t)row0 * K;
+    const int share_lds = (loads_w ? 0 : DT * TK) + row0 * TK;
+    const bool whole = rows_left >= 64;                        /* wave-uniform */
+    uint32_t lane_off[2];                                      /* bytes from the first row of a piece, by parity of the piece */
+#pragma unroll
+    for (int par = 0; par < 2; par++)
+        lane_off[par] = (uint32_t)((lane >> 3) * K + 8 * ((lane & 7) ^ ((4 * par + (lane >> 4)) & 7))) * 2u;
+    auto request = [&](int kt, int stage) {
+        uint16_t *dst = dlds + stage * DSTAGE + share_lds;
+        if (whole) {
+            const uint16_t *src = share + (size_t)kt * TK;
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                             ::"s"(lds_address(dst + 8 * j * TK)), "v"(lane_off[j & 1]), "s"(src + (size_t)(8 * j) * K) : "memory");
+        } else {
+            /* rows past the end of the matrix are redirected to its last row (their outputs are never stored) */
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int r = 8 * j + (lane >> 3);
+                const int chunk = (lane & 7) ^ ((r >> 1) & 7);
+                const int rr = min(r, rows_left - 1);             /* rows_left <= 0: before the share, still inside the matrix */
+                const uint16_t *src = share + (ptrdiff_t)rr * K + (size_t)kt * TK + 8 * chunk;
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                             ::"s"(lds_address(dst + 8 * j * TK)), "v"(src) : "memory");
+            }
+        }
+    };
+
+    f32x4 acc[4][8];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 8; b++) acc[a][b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    /* operand addresses inside a stage (elements): W rows n = 64 wn + 16 a + li, x rows m = 128 wm + 16 b + li;
+     * (row >> 1) & 7 = li >> 1 for both, whatever a or b */
+    int a_rd[2], b_rd[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        const int slot = 8 * ((4 * ks + lg) ^ (li >> 1));
+        a_rd[ks] = (64 * wn + li) * TK + slot;
+        b_rd[ks] = DT * TK + (128 * wm + li) * TK + slot;
+    }
+    const int nk = K / TK;
+
+    request(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    lds_barrier();
+
+    for (int kt = 0; kt < nk; kt++) {
+        const uint16_t *cur = dlds + (kt & 1) * DSTAGE;
+        /* Four quarters per k tile: k-step ks, x blocks 4 half .. +3. The operands of the next quarter are
+         * requested from LDS before the 16 MFMAs of this one are issued, so that the LDS works while the
+         * matrix core does; the W operands of a k-step are read with its first quarter. */
+        u32x4 av[2][4], bv[2][4];
+        auto read_quarter = [&](int qi) {
+            const int ks = qi >> 1, half = qi & 1;
+            if (half == 0) {
+#pragma unroll
+                for (int a = 0; a < 4; a++) av[ks][a] = *reinterpret_cast<const u32x4 *>(&cur[a_rd[ks] + 16 * a * TK]);
+            }
+#pragma unroll
+            for (int b = 0; b < 4; b++) bv[qi & 1][b] = *reinterpret_cast<const u32x4 *>(&cur[b_rd[ks] + 16 * (4 * half + b) * TK]);
+        };
+        read_quarter(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int qi = 0; qi < 4; qi++) {
+            if (qi < 3) read_quarter(qi + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            const int ks = qi >> 1, half = qi & 1;
+#pragma unroll
+            for (int a = 0; a < 4; a++)
+#pragma unroll
+                for (int b = 0; b < 4; b++)
+                    acc[a][4 * half + b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, av[ks][a]), __builtin_bit_cast(bf16x8, bv[qi & 1][b]), acc[a][4 * half + b], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            /* the next k tile: HBM/L2 -> the other stage, whose last readers passed the barrier that ended
+             * tile kt - 1. Requested behind the first quarter's MFMAs rather than right after the barrier,
+             * where every wave would issue its requests before its first operand read. */
+            if (qi == 0 && kt + 1 < nk) { request(kt + 1, (kt + 1) & 1); __builtin_amdgcn_sched_barrier(0); }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       /* this wave's share of the next tile has landed */
+        lds_barrier();                                          /* everybody's has, and nobody reads this tile any more */
+    }
+
+    /* acc[a][b][r] = y[m0 + 128 wm + 16 b + li][n0 + 64 wn + 16 a + 4 lg + r].
+     * Stored straight from the accumulators a store instruction covers 16 rows x 64 (f32) or 32 (bf16) bytes,
+     * and the write path is bound by the number of such pieces, not by bytes. So the wave's 128 x 64 block
+     * goes through LDS (free after the loop's last barrier; 16 KB per wave, its own region, no workgroup
+     * barrier) and leaves as 16 B per lane along the rows: 4 rows x 256 B (f32) or 8 rows x 128 B (bf16) per
+     * instruction. 16 B chunk c of row r sits in slot c ^ (r mod 16) (f32, 16 chunks a row) or
+     * c ^ (r mod 8) (bf16, 8 chunks), which keeps both the writes and the reads off each other's banks.
+     * LDS serves a wave's instructions in order, so the reads see the writes without a barrier. */
+    constexpr int PER16 = 16 / (int)sizeof(OUT);               /* outputs per 16 B */
+    const bool staged = N % PER16 == 0 && ((uintptr_t)y & 15) == 0;
+    if (staged) {
+        uint16_t *mine = dlds + wave * 8192;                    /* 16 KB */
+        const int mw = m0 + 128 * wm, nw = n0 + 64 * wn;
+        if constexpr (sizeof(OUT) == 4) {
+            float *buf = reinterpret_cast<float *>(mine);       /* 64 rows x 64 f32, half of the block at a time */
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+#pragma unroll
+                for (int bb = 0; bb < 4; bb++)
+#pragma unroll
+                    for (int a = 0; a < 4; a++)
+                        *reinterpret_cast<f32x4 *>(&buf[(16 * bb + li) * 64 + 4 * ((4 * a + lg) ^ li)]) = acc[a][4 * half + bb];
+#pragma unroll
+                for (int it = 0; it < 16; it++) {
+                    const int row = 4 * it + (lane >> 4), c = lane & 15;
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(&buf[row * 64 + 4 * (c ^ (row & 15))]);
+                    const int m = mw + 64 * half + row, n = nw + 4 * c;
+                    if (m < M && n < N) *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(y) + (size_t)m * N + n) = v;
+                }
+            }
+        } else {
+            uint16_t *buf = mine;                               /* 128 rows x 64 bf16 */
+#pragma unroll
+            for (int b = 0; b < 8; b++)
+#pragma unroll
+                for (int a = 0; a < 4; a++) {
+                    const int chunk = 2 * a + (lg >> 1);
+                    *reinterpret_cast<uint2 *>(&buf[(16 * b + li) * 64 + 8 * (chunk ^ (li & 7)) + 4 * (lg & 1)]) =
+                        make_uint2(pack_bf16(acc[a][b][0], acc[a][b][1]), pack_bf16(acc[a][b][2], acc[a][b][3]));
+                }
+#pragma unroll
+            for (int it = 0; it < 16; it++) {
+                const int row = 8 * it + (lane >> 3), c = lane & 7;
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(&buf[row * 64 + 8 * (c ^ (row & 7))]);
+                const int m = mw + row, n = nw + 8 * c;
+                if (m < M && n < N) *reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(y) + (size_t)m * N + n) = v;
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+        const int m = m0 + 128 * wm + 16 * b + li;
+        if (m >= M) continue;
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            const int n = n0 + 64 * wn + 16 * a + 4 * lg;
+            if (n < N) store4(y + (size_t)m * N + n, acc[a][b], N - n);
+        }
+    }
+}
+
 /* Any K / alignment: one thread per output element. */
 template <typename OUT>
 __global__ void __launch_bounds__(256)
@@ -165,7 +360,22 @@ k_gemm_scalar(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_
 template <typename OUT>
 int gemm(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, int N, int K) {
     if (M <= 0 || N <= 0) return 0;
-    if (K > 0 && K % 8 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)W & 15) == 0) {
+    const bool aligned16 = ((uintptr_t)x & 15) == 0 && ((uintptr_t)W & 15) == 0;
+    if (K > 0 && K % TK == 0 && aligned16 && M >= DT && N >= DT && (size_t)K * 2 * 8 < ((size_t)1 << 31)) {
+        static bool configured[2] = {false, false};
+        constexpr int which = sizeof(OUT) == 4 ? 0 : 1;
+        constexpr int lds_bytes = 2 * DSTAGE * (int)sizeof(uint16_t);
+        if (!configured[which]) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_dma<OUT>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+            if (e != hipSuccess) return (int)e;
+            configured[which] = true;
+        }
+        const int tiles_m = (M + DT - 1) / DT, tiles_n = (N + DT - 1) / DT, total = tiles_m * tiles_n;
+        const int per_xcd = (total + 7) / 8;
+        hipLaunchKernelGGL((k_gemm_dma<OUT>), dim3((unsigned)per_xcd * 8), dim3(512), lds_bytes, st, y, x, W, M, N, K,
+                           tiles_m, total, per_xcd);
+    } else if (K > 0 && K % 8 == 0 && aligned16) {
         /* 2 x 2 waves (128 x 128 tiles) measured best on the transformer shapes: 4 x 2 and 2 x 4 are
          * 5-8 % slower on the wide projections, 4 x 1 and 2 x 1 15-30 % slower. */
         constexpr int WM = 2, WN = 2, TM = 64 * WM, TN = 64 * WN;
