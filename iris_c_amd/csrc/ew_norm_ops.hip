@@ -259,84 +259,151 @@ int launch_row_norm(hipStream_t st, uint16_t *out_bf, float *xres, const float *
     return (int)hipGetLastError();
 }
 
-/* ---------------------------------------------------------------- group norm */
+/* ---------------------------------------------------------------- group norm
+ *
+ * Two passes over the image in all: one for the statistics, one that normalises.
+ *
+ * Statistics in ONE pass: a thread sums (x - K) and (x - K)^2 over its share of a group, K being
+ * the first value it reads. K is a sample of the data, so the sums stay of the size of the
+ * spread and the cancellation that plain sum / sum-of-squares formulas suffer does not arise.
+ * Each thread's (count, mean, M2) is then merged with the others' by the pairwise update of the
+ * parallel variance algorithm: inside the workgroup in f32, across workgroups in double.
+ * (The reference reads the image twice for the statistics, mean first and then the squared
+ * deviations, iris_cuda.cu:1069-1074; the merged single pass gives the same moments to f32
+ * rounding.) */
 
-constexpr int GN_BLOCKS = 256;       /* partial sums per group */
+constexpr int GN_MAX_BLOCKS = 1024;      /* partial moments per group */
 
-/* part[g * GN_BLOCKS + b] = sum over block b's pixels of group g of x (mean == NULL) or of
- * (x - mean[g])^2. Coalesced form: needs c % 4 == 0, cg % 4 == 0 and (c / 4) dividing 256;
- * a thread keeps one quad of channels, the workgroup walks 256 / (c / 4) pixels per step. */
+struct Moments { float n, mean, m2; };
+
+__device__ __forceinline__ void merge(Moments &a, const Moments b) {
+    if (b.n == 0.0f) return;
+    const float n = a.n + b.n, d = b.mean - a.mean;
+    a.mean += d * (b.n / n);
+    a.m2 += b.m2 + d * d * (a.n * b.n / n);
+    a.n = n;
+}
+
+/* from sums shifted by k */
+__device__ __forceinline__ Moments from_shifted(float n, float k, float s, float ss) {
+    Moments m = {n, 0.0f, 0.0f};
+    if (n > 0.0f) { m.mean = k + s / n; m.m2 = fmaxf(ss - s * s / n, 0.0f); }
+    return m;
+}
+
+/* part[(g * nblocks + b)] = moments of group g over the pixels of block b. Coalesced form: needs
+ * c % 4 == 0, cg % 4 == 0 and (c / 4) dividing 256; a thread keeps one quad of channels (inside
+ * one group), the workgroup walks 256 / (c / 4) pixels per step with 16-byte loads. */
 __global__ void __launch_bounds__(ROW_THREADS)
-k_gn_partial_rows(float *__restrict__ part, const float *__restrict__ in, const float *__restrict__ mean,
-                  int hw, int c, int cg) {
-    __shared__ float sh[ROW_THREADS];
+k_gn_moments_quads(Moments *__restrict__ part, const float *__restrict__ in, int hw, int c, int cg, int per_block) {
+    __shared__ Moments sh[ROW_THREADS];
     const int quads = c >> 2, ppi = ROW_THREADS / quads;      /* pixels per iteration */
     const int q = threadIdx.x % quads, sub = threadIdx.x / quads;
-    const int g = (4 * q) / cg;
-    const float m = mean ? mean[g] : 0.0f;
-    const int per_block = (hw + GN_BLOCKS - 1) / GN_BLOCKS;
     const int start = blockIdx.x * per_block, end = min(start + per_block, hw);
-    float s = 0.0f;
-    for (int p = start + sub; p < end; p += ppi) {
+    float n = 0.0f, k = 0.0f, s = 0.0f, ss = 0.0f;
+    int p = start + sub;
+    if (p < end) k = in[(size_t)p * c + 4 * q];
+    for (; p < end; p += ppi) {
         const float4 v = *reinterpret_cast<const float4 *>(in + (size_t)p * c + 4 * q);
-        if (mean) s += ((v.x - m) * (v.x - m) + (v.y - m) * (v.y - m)) + ((v.z - m) * (v.z - m) + (v.w - m) * (v.w - m));
-        else s += (v.x + v.y) + (v.z + v.w);
+        const float a0 = v.x - k, a1 = v.y - k, a2 = v.z - k, a3 = v.w - k;
+        s += (a0 + a1) + (a2 + a3);
+        ss += (a0 * a0 + a1 * a1) + (a2 * a2 + a3 * a3);
+        n += 4.0f;
     }
-    sh[threadIdx.x] = s;
+    sh[threadIdx.x] = from_shifted(n, k, s, ss);
     __syncthreads();
     const int groups = c / cg, qpg = cg >> 2;
     if ((int)threadIdx.x < groups) {
-        float t = 0.0f;
+        Moments t = {0.0f, 0.0f, 0.0f};
         for (int sb = 0; sb < ppi; sb++)
-            for (int j = 0; j < qpg; j++) t += sh[sb * quads + threadIdx.x * qpg + j];
-        part[(size_t)threadIdx.x * GN_BLOCKS + blockIdx.x] = t;
+            for (int j = 0; j < qpg; j++) merge(t, sh[sb * quads + threadIdx.x * qpg + j]);
+        part[(size_t)threadIdx.x * gridDim.x + blockIdx.x] = t;
     }
 }
 
-/* Any shape: one workgroup per (group, block), strided reads. */
+/* Any shape: one workgroup per (group, block), scalar strided reads. */
 __global__ void __launch_bounds__(ROW_THREADS)
-k_gn_partial(float *__restrict__ part, const float *__restrict__ in, const float *__restrict__ mean,
-             int hw, int c, int cg) {
-    __shared__ float sh[4];
+k_gn_moments_any(Moments *__restrict__ part, const float *__restrict__ in, int hw, int c, int cg) {
+    __shared__ Moments sh[ROW_THREADS];
     const int g = blockIdx.x, b = blockIdx.y;
-    const size_t n = (size_t)hw * cg;
-    const size_t per_block = (n + GN_BLOCKS - 1) / GN_BLOCKS;
-    const size_t start = (size_t)b * per_block, end = start + per_block < n ? start + per_block : n;
-    const float m = mean ? mean[g] : 0.0f;
-    float s = 0.0f;
+    const size_t total = (size_t)hw * cg;
+    const size_t per_block = (total + gridDim.y - 1) / gridDim.y;
+    const size_t start = (size_t)b * per_block, end = start + per_block < total ? start + per_block : total;
+    float n = 0.0f, k = 0.0f, s = 0.0f, ss = 0.0f;
     for (size_t i = start + threadIdx.x; i < end; i += ROW_THREADS) {
         const float v = in[(i / cg) * c + (size_t)g * cg + i % cg];
-        s += mean ? (v - m) * (v - m) : v;
+        if (n == 0.0f) k = v;
+        const float a = v - k;
+        s += a; ss += a * a; n += 1.0f;
     }
-    s = block_sum(s, sh);
-    if (threadIdx.x == 0) part[(size_t)g * GN_BLOCKS + b] = s;
+    sh[threadIdx.x] = from_shifted(n, k, s, ss);
+    __syncthreads();
+    for (int half = ROW_THREADS / 2; half > 0; half >>= 1) {
+        if ((int)threadIdx.x < half) merge(sh[threadIdx.x], sh[threadIdx.x + half]);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) part[(size_t)g * gridDim.y + b] = sh[0];
 }
 
-/* stats[g] = mean (pass 0) or stats[groups + g] = 1 / sqrt(var + eps) (pass 1), in double */
-__global__ void k_gn_finalize(float *__restrict__ stats, const float *__restrict__ part, int groups,
-                              double count, float eps, int pass) {
-    const int g = blockIdx.x * blockDim.x + threadIdx.x;
-    if (g >= groups) return;
-    double s = 0.0;
-    for (int b = 0; b < GN_BLOCKS; b++) s += (double)part[(size_t)g * GN_BLOCKS + b];
-    if (pass == 0) stats[g] = (float)(s / count);
-    else stats[groups + g] = (float)(1.0 / sqrt(s / count + (double)eps));
+/* stats[g] = mean, stats[groups + g] = 1 / sqrt(var + eps): the partial moments merged in double, one
+ * wave per group (each lane merges its share of the workgroups' partials, then the lanes merge pairwise) */
+__device__ __forceinline__ void merge64(double &n, double &mean, double &m2, double nb, double mb, double m2b) {
+    if (nb == 0.0) return;
+    const double tot = n + nb, d = mb - mean;
+    mean += d * (nb / tot);
+    m2 += m2b + d * d * (n * nb / tot);
+    n = tot;
 }
 
+__global__ void __launch_bounds__(64)
+k_gn_finish(float *__restrict__ stats, const Moments *__restrict__ part, int groups, int nblocks, float eps) {
+    const int g = blockIdx.x, lane = threadIdx.x;
+    double n = 0.0, mean = 0.0, m2 = 0.0;
+    for (int b = lane; b < nblocks; b += 64) {
+        const Moments m = part[(size_t)g * nblocks + b];
+        merge64(n, mean, m2, (double)m.n, (double)m.mean, (double)m.m2);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const double nb = __shfl_xor(n, off, 64), mb = __shfl_xor(mean, off, 64), m2b = __shfl_xor(m2, off, 64);
+        /* both partners must end with the same value: merge in a fixed order (lower lane first) */
+        double n0 = n, mean0 = mean, m20 = m2, n1 = nb, mean1 = mb, m21 = m2b;
+        if (lane & off) { n0 = nb; mean0 = mb; m20 = m2b; n1 = n; mean1 = mean; m21 = m2; }
+        merge64(n0, mean0, m20, n1, mean1, m21);
+        n = n0; mean = mean0; m2 = m20;
+    }
+    if (lane == 0) {
+        stats[g] = (float)mean;
+        stats[groups + g] = (float)(1.0 / sqrt((n > 0.0 ? m2 / n : 0.0) + (double)eps));
+    }
+}
+
+/* out = (x - mean[g]) * rstd[g] * gamma[ch] + beta[ch], optionally through SiLU. VEC = 4: a thread's four
+ * channels are one aligned quad, which lies inside one group (c % 4 == 0 and cg % 4 == 0) or, when
+ * cg % 4 != 0, is looked up channel by channel. */
 template <int VEC>
 __global__ void __launch_bounds__(EW_THREADS)
-k_gn_apply(float *__restrict__ out, const float *__restrict__ in, const float *__restrict__ stats,
-           const float *__restrict__ gamma, const float *__restrict__ beta, int c, int cg, int groups,
-           int do_silu, size_t n) {
+k_gn_normalize(float *__restrict__ out, const float *__restrict__ in, const float *__restrict__ stats,
+               const float *__restrict__ gamma, const float *__restrict__ beta, int c, int cg, int groups,
+               int do_silu, size_t n) {
     const size_t i = ((size_t)blockIdx.x * EW_THREADS + threadIdx.x) * VEC;
     if (i >= n) return;
-    float v[VEC];
-    if (VEC == 4) *reinterpret_cast<float4 *>(v) = *reinterpret_cast<const float4 *>(in + i);
-    else v[0] = in[i];
+    const int ch0 = (int)(i % (size_t)c);
+    float v[VEC], ga[VEC], be[VEC];
+    if (VEC == 4) {
+        *reinterpret_cast<float4 *>(v) = *reinterpret_cast<const float4 *>(in + i);
+        *reinterpret_cast<float4 *>(ga) = *reinterpret_cast<const float4 *>(gamma + ch0);
+        *reinterpret_cast<float4 *>(be) = *reinterpret_cast<const float4 *>(beta + ch0);
+    } else {
+        v[0] = in[i]; ga[0] = gamma[ch0]; be[0] = beta[ch0];
+    }
+    const bool one_group = VEC == 1 || cg % 4 == 0;
+    const int g0 = ch0 / cg;
+    const float mean0 = stats[g0], rstd0 = stats[groups + g0];
 #pragma unroll
     for (int j = 0; j < VEC; j++) {
-        const int ch = (int)((i + j) % c), g = ch / cg;
-        const float y = (v[j] - stats[g]) * stats[groups + g] * gamma[ch] + beta[ch];
+        float mean = mean0, rstd = rstd0;
+        if (!one_group) { const int g = (ch0 + j) / cg; mean = stats[g]; rstd = stats[groups + g]; }
+        const float y = (v[j] - mean) * rstd * ga[j] + be[j];
         v[j] = do_silu ? silu(y) : y;
     }
     if (VEC == 4) *reinterpret_cast<float4 *>(out + i) = *reinterpret_cast<float4 *>(v);
@@ -407,31 +474,37 @@ int iris_hip_rms_norm_residual(void *stream, float *x, const float *a, const flo
     return launch_row_norm<RMS_NORM_RESIDUAL>((hipStream_t)stream, nullptr, x, a, w, gate, rows, dim, eps);
 }
 
-size_t iris_hip_group_norm_scratch_floats(int groups) { return (size_t)groups * GN_BLOCKS + 2 * (size_t)groups; }
+size_t iris_hip_group_norm_scratch_floats(int groups) { return 3 * (size_t)groups * GN_MAX_BLOCKS + 2 * (size_t)groups; }
 
 /* scratch: iris_hip_group_norm_scratch_floats(groups) floats of device memory */
 int iris_hip_group_norm(void *stream, float *scratch, float *out, const float *in, const float *gamma,
                         const float *beta, int hw, int c, int groups, float eps, int do_silu) {
     if (hw <= 0 || c <= 0) return 0;
     hipStream_t st = (hipStream_t)stream;
-    float *part = scratch, *stats = scratch + (size_t)groups * GN_BLOCKS;
+    Moments *part = reinterpret_cast<Moments *>(scratch);
+    float *stats = scratch + 3 * (size_t)groups * GN_MAX_BLOCKS;
     const int cg = c / groups;
-    const double count = (double)hw * cg;
-    const bool rows_form = c % 4 == 0 && cg % 4 == 0 && c / 4 <= ROW_THREADS && ROW_THREADS % (c / 4) == 0 && al16(in);
-    for (int pass = 0; pass < 2; pass++) {
-        if (rows_form)
-            hipLaunchKernelGGL(k_gn_partial_rows, dim3(GN_BLOCKS), dim3(ROW_THREADS), 0, st, part, in,
-                               pass ? stats : (const float *)nullptr, hw, c, cg);
-        else
-            hipLaunchKernelGGL(k_gn_partial, dim3(groups, GN_BLOCKS), dim3(ROW_THREADS), 0, st, part, in,
-                               pass ? stats : (const float *)nullptr, hw, c, cg);
-        hipLaunchKernelGGL(k_gn_finalize, dim3(blocks_for(groups, 64)), dim3(64), 0, st, stats, part, groups, count, eps, pass);
+    const bool quads_form = c % 4 == 0 && cg % 4 == 0 && c / 4 <= ROW_THREADS && ROW_THREADS % (c / 4) == 0 && al16(in);
+    int nblocks;
+    if (quads_form) {
+        const int ppi = ROW_THREADS / (c / 4);
+        nblocks = (hw + ppi - 1) / ppi;                         /* at least one step of the workgroup per block */
+        if (nblocks > GN_MAX_BLOCKS) nblocks = GN_MAX_BLOCKS;
+        const int per_block = (hw + nblocks - 1) / nblocks;
+        nblocks = (hw + per_block - 1) / per_block;
+        hipLaunchKernelGGL(k_gn_moments_quads, dim3(nblocks), dim3(ROW_THREADS), 0, st, part, in, hw, c, cg, per_block);
+    } else {
+        const size_t total = (size_t)hw * cg;
+        nblocks = (int)((total + 4 * ROW_THREADS - 1) / (4 * ROW_THREADS));
+        if (nblocks > GN_MAX_BLOCKS) nblocks = GN_MAX_BLOCKS;
+        hipLaunchKernelGGL(k_gn_moments_any, dim3(groups, nblocks), dim3(ROW_THREADS), 0, st, part, in, hw, c, cg);
     }
+    hipLaunchKernelGGL(k_gn_finish, dim3(groups), dim3(64), 0, st, stats, part, groups, nblocks, eps);
     const size_t n = (size_t)hw * c;
-    if (al16(out) && al16(in) && c % 4 == 0)
-        hipLaunchKernelGGL(k_gn_apply<4>, dim3(blocks_for(n, EW_THREADS * 4)), dim3(EW_THREADS), 0, st, out, in, stats, gamma, beta, c, cg, groups, do_silu, n);
+    if (al16(out) && al16(in) && al16(gamma) && al16(beta) && c % 4 == 0)
+        hipLaunchKernelGGL(k_gn_normalize<4>, dim3(blocks_for(n, EW_THREADS * 4)), dim3(EW_THREADS), 0, st, out, in, stats, gamma, beta, c, cg, groups, do_silu, n);
     else
-        hipLaunchKernelGGL(k_gn_apply<1>, dim3(blocks_for(n, EW_THREADS)), dim3(EW_THREADS), 0, st, out, in, stats, gamma, beta, c, cg, groups, do_silu, n);
+        hipLaunchKernelGGL(k_gn_normalize<1>, dim3(blocks_for(n, EW_THREADS)), dim3(EW_THREADS), 0, st, out, in, stats, gamma, beta, c, cg, groups, do_silu, n);
     return (int)hipGetLastError();
 }
 

@@ -208,6 +208,20 @@ def test_group_norm(dev, orc, hw, c, groups, silu):
     np.testing.assert_allclose(got, orc.dev_group_norm(img, gamma, beta, groups, 1e-6, silu), atol=2e-5)
 
 
+@pytest.mark.parametrize("hw,c,groups", [(70000, 128, 32), (5000, 512, 32), (3001, 6, 3), (1, 8, 2)])
+def test_group_norm_single_pass_statistics_far_from_zero(dev, orc, hw, c, groups):
+    """The statistics are taken in one pass with shifted sums and merged moments; data with a mean of 100
+    standard deviations is where a careless one-pass formula loses everything. More workgroups than
+    the partial-moment table has rows (70000 pixels), many channels per group, the scalar path, one pixel."""
+    img = rnd((hw, c), hw + c, 0.5) + 50.0 + np.arange(c, dtype=np.float32)[None, :] * 0.01
+    gamma, beta = 1 + rnd(c, 1, 0.1), rnd(c, 2, 0.1)
+    dimg, dg, db = dev.put(img), dev.put(gamma), dev.put(beta)
+    dout = dev.alloc(hw * c * 4)
+    got = run(dev, lambda: dev.lib.iris_dev_group_norm(dout, dimg, dg, db, hw, c, groups, 1e-6, 0), [(dout, (hw, c), np.float32)])
+    want = orc.dev_group_norm(img, gamma, beta, groups, 1e-6, 0)
+    np.testing.assert_allclose(got, want, atol=2e-4)
+
+
 @pytest.mark.parametrize("h,w,c", [(3, 4, 5), (16, 16, 128)])
 def test_upsample2x(dev, orc, h, w, c):
     img = rnd((h * w, c), c)
