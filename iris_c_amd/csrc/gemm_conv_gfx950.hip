@@ -25,9 +25,11 @@
  * of 8 with 16-byte aligned rows, otherwise the scalar kernel below takes over (the
  * only such caller is the 3-channel input convolution of the VAE encoder).
  *
- * Convolution = gather of the k x k input patches as bf16 rows (what the reference
- * does, iris_cuda.cu:959-985) into scratch, then the same GEMM, chunked by output
- * pixels so the scratch stays bounded.
+ * Convolution with a multiple of 64 input channels (every layer of the VAE but its first) is an
+ * implicit GEMM: the image is converted to bf16 once and k_gemm_dma fetches the pixels under each
+ * tap itself, so the k x k patches are never written out. Other shapes gather the patches as bf16
+ * rows into scratch (what the reference does for all of them, iris_cuda.cu:959-985) and run the
+ * plain GEMM on them, chunked by output pixels so the scratch stays bounded.
  */
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -151,15 +153,15 @@ k_gemm_bf16(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t 
     }
 }
 
-/* ---- the large-shape kernel: 256 x 256 tiles, 8 waves, tiles straight from HBM/L2 into LDS ----
+/* ---- the large-shape kernel: 256 x TN tiles, 8 waves, tiles straight from HBM/L2 into LDS ----
  *
- * For M, N >= 256 and K a multiple of 64. A workgroup is 8 waves (two per SIMD, one workgroup per
- * CU), 2 along m x 4 along n, each wave owning 128 (m) x 64 (n) outputs = 8 x 4 accumulator
- * blocks: 12 operand reads from LDS feed 32 MFMAs per k-step. K advances in tiles of 64; a stage
- * holds the W tile (256 rows of 128 B) and the x tile (256 rows), 64 KB, two stages. The tiles
- * are written by global_load_lds_dwordx4 (64 lanes x 16 B = eight 128 B rows per instruction,
- * no registers, no LDS-write instructions), 8 such loads per wave and k tile (waves 0-3 the W
- * rows, 4-7 the x rows), requested one k tile ahead; one barrier per k tile.
+ * For M >= 256, N >= TN (256 or 128) and K a multiple of 64. A workgroup is 8 waves (two per SIMD,
+ * one workgroup per CU). TN = 256: 2 waves along m x 4 along n, each wave owning 128 (m) x 64 (n)
+ * outputs = 8 x 4 accumulator blocks, 12 operand reads from LDS per 32 MFMAs. TN = 128: 4 x 2
+ * waves of 64 x 64 (8 reads per 16 MFMAs). K advances in tiles of 64; a stage holds the W tile
+ * (TN rows of 128 B) and the x tile (256 rows), two stages. The tiles are written by
+ * global_load_lds_dwordx4 (64 lanes x 16 B = eight 128 B rows per instruction, no registers, no
+ * LDS-write instructions), requested one k tile ahead; one barrier per k tile.
  *
  * Direct loads cannot pad rows, so the 16 B chunk c of tile row r is kept in slot
  * c ^ ((r >> 1) & 7) of its row, the permutation applied to the source address of the lane that
@@ -167,75 +169,133 @@ k_gemm_bf16(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t 
  * with chunk c0 and eight with c0 + 1, and of each parity of row four with either. Two
  * consecutive rows span the 64 banks once, so rows of equal parity must differ in slot: the
  * rows with chunk c0 have (r >> 1) & 7 in {0, 1, 6, 7} (or {2, 3, 4, 5}), those with c0 + 1 the
- * complement, and c0 is a multiple of 2, which makes the eight slots distinct. */
-constexpr int DT = 256;                          /* tile edge (m and n) */
-constexpr int DSTAGE = 2 * DT * TK;              /* elements per stage: W tile then x tile */
+ * complement, and c0 is a multiple of 2, which makes the eight slots distinct.
+ *
+ * CONV: the same product with x never materialised ("implicit GEMM"). Row m of x is output pixel
+ * p0 + m, column (tap, channel) is the input pixel under that tap: the 128 B a lane group fetches
+ * for (row, k tile) are 64 consecutive channels of ONE input pixel (cin is a multiple of 64, so a
+ * k tile never straddles taps), found from the pixel's coordinates; taps that fall outside the
+ * image read a page of zeros instead. The image is bf16, channels last. The bias is added in the
+ * epilogue. */
+constexpr int DT = 256;                          /* tile rows of x (m) */
+
+struct ConvGeom {
+    int h, w, cin, ksz, stride, pad, ow, p0;     /* input size, kernel, output width, first output pixel of this launch */
+    const uint16_t *zeros;                       /* >= 128 B of zeros, 16-byte aligned */
+    const float *bias;                           /* [N] or null; 16-byte aligned */
+};
 
 __device__ __forceinline__ uint32_t lds_address(const uint16_t *p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
 }
 
-template <typename OUT>
+template <typename OUT, int TN, bool CONV>
 __global__ void __launch_bounds__(512, 2)
 k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *__restrict__ W,
-           int M, int N, int K, int tiles_m, int total, int per_xcd) {
-    extern __shared__ __align__(16) uint16_t dlds[];          /* two stages */
+           int M, int N, int K, int tiles_m, int total, int per_xcd, ConvGeom geo) {
+    constexpr int WAVES_N = TN / 64, WAVES_M = 8 / WAVES_N;    /* wave grid */
+    constexpr int NB = DT / WAVES_M / 16;                      /* x blocks (16 rows) per wave: 8 or 4 */
+    constexpr int HALVES = NB / 4;
+    constexpr int W_PIECES = TN / 64, X_PIECES = 4;            /* 8-row pieces per wave and k tile */
+    constexpr int STAGE = (TN + DT) * TK;                      /* elements: W tile then x tile */
+    extern __shared__ __align__(16) uint16_t dlds[];          /* two stages (and room for the epilogue) */
     /* each XCD (own L2) walks a contiguous range of the tile list, m fastest: neighbours share a W tile */
     const int work = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (work >= total) return;
     const int bm = work % tiles_m, bn = work / tiles_m;
-    const int m0 = bm * DT, n0 = bn * DT;
+    const int m0 = bm * DT, n0 = bn * TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
-    const int wm = wave & 1, wn = wave >> 1;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
 
-    /* this wave's share of a stage: rows 64 (wave % 4) .. +63 of the W tile (waves 0-3) or the x tile */
-    const bool loads_w = wave < 4;
-    const int row0 = 64 * (wave & 3);                          /* first row of the share inside its tile */
-    const int rows_left = (loads_w ? N - n0 : M - m0) - row0;  /* rows of the share that exist (may be <= 0) */
-    const uint16_t *share = (loads_w ? W + (size_t)n0 * K : x + (size_t)m0 * K) + (size_t)row0 * K;
-    const int share_lds = (loads_w ? 0 : DT * TK) + row0 * TK;
-    const bool whole = rows_left >= 64;                        /* wave-uniform */
-    uint32_t lane_off[2];                                      /* bytes from the first row of a piece, by parity of the piece */
+    /* this wave's share of a stage: W rows 8 W_PIECES wave .. and x rows 32 wave .. +31 */
+    const int w_row0 = 8 * W_PIECES * wave, x_row0 = 8 * X_PIECES * wave;
+    const int w_left = N - n0 - w_row0, x_left = M - m0 - x_row0;    /* rows of the share that exist (may be <= 0) */
+    const uint16_t *w_share = W + (size_t)n0 * K + (size_t)w_row0 * K;
+    const uint16_t *x_share = CONV ? x : x + (size_t)m0 * K + (size_t)x_row0 * K;
+    /* byte offset of this lane's 16 B inside a piece, from the piece's first row, by parity of the piece:
+     * row lane / 8, chunk (lane % 8) ^ swizzle of that row */
+    uint32_t lane_off[2];
+    int lane_chunk[2];
 #pragma unroll
-    for (int par = 0; par < 2; par++)
-        lane_off[par] = (uint32_t)((lane >> 3) * K + 8 * ((lane & 7) ^ ((4 * par + (lane >> 4)) & 7))) * 2u;
+    for (int par = 0; par < 2; par++) {
+        lane_chunk[par] = (lane & 7) ^ ((4 * par + (lane >> 4)) & 7);
+        lane_off[par] = (uint32_t)((lane >> 3) * K + 8 * lane_chunk[par]) * 2u;
+    }
+    /* CONV: coordinates of the four output pixels whose rows this lane fetches (piece j: row 8 j + lane / 8) */
+    int pix_y[X_PIECES], pix_x[X_PIECES];
+    if (CONV) {
+#pragma unroll
+        for (int j = 0; j < X_PIECES; j++) {
+            const int r = x_row0 + 8 * j + (lane >> 3);
+            const int p = geo.p0 + min(m0 + r, M - 1);
+            const int oy = p / geo.ow;
+            pix_y[j] = oy * geo.stride - geo.pad;
+            pix_x[j] = (p - oy * geo.ow) * geo.stride - geo.pad;
+        }
+    }
+    auto load16 = [&](uint16_t *dst, const uint16_t *src) {     /* per-lane source address */
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                     ::"s"(lds_address(dst)), "v"(src) : "memory");
+    };
     auto request = [&](int kt, int stage) {
-        uint16_t *dst = dlds + stage * DSTAGE + share_lds;
-        if (whole) {
-            const uint16_t *src = share + (size_t)kt * TK;
+        uint16_t *w_dst = dlds + stage * STAGE + w_row0 * TK;
+        uint16_t *x_dst = dlds + stage * STAGE + TN * TK + x_row0 * TK;
+        if (w_left >= 8 * W_PIECES) {                           /* wave-uniform */
+            const uint16_t *src = w_share + (size_t)kt * TK;
 #pragma unroll
-            for (int j = 0; j < 8; j++)
+            for (int j = 0; j < W_PIECES; j++)
                 asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                             ::"s"(lds_address(dst + 8 * j * TK)), "v"(lane_off[j & 1]), "s"(src + (size_t)(8 * j) * K) : "memory");
+                             ::"s"(lds_address(w_dst + 8 * j * TK)), "v"(lane_off[j & 1]), "s"(src + (size_t)(8 * j) * K) : "memory");
         } else {
             /* rows past the end of the matrix are redirected to its last row (their outputs are never stored) */
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int r = 8 * j + (lane >> 3);
-                const int chunk = (lane & 7) ^ ((r >> 1) & 7);
-                const int rr = min(r, rows_left - 1);             /* rows_left <= 0: before the share, still inside the matrix */
-                const uint16_t *src = share + (ptrdiff_t)rr * K + (size_t)kt * TK + 8 * chunk;
-                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                             ::"s"(lds_address(dst + 8 * j * TK)), "v"(src) : "memory");
+            for (int j = 0; j < W_PIECES; j++) {
+                const int rr = min(8 * j + (lane >> 3), w_left - 1);
+                load16(w_dst + 8 * j * TK, w_share + (ptrdiff_t)rr * K + (size_t)kt * TK + 8 * lane_chunk[j & 1]);
+            }
+        }
+        if (CONV) {
+            const int per_tap = geo.cin / TK;                   /* k tiles per tap */
+            const int tap = kt / per_tap, c0 = (kt - tap * per_tap) * TK;
+            const int ky = tap / geo.ksz, kx = tap - ky * geo.ksz;
+#pragma unroll
+            for (int j = 0; j < X_PIECES; j++) {
+                const int iy = pix_y[j] + ky, ix = pix_x[j] + kx;
+                const bool inside = iy >= 0 && iy < geo.h && ix >= 0 && ix < geo.w;
+                const uint16_t *src = inside ? x + ((size_t)iy * geo.w + ix) * geo.cin + c0 + 8 * lane_chunk[j & 1]
+                                             : geo.zeros + 8 * (lane & 7);
+                load16(x_dst + 8 * j * TK, src);
+            }
+        } else if (x_left >= 8 * X_PIECES) {
+            const uint16_t *src = x_share + (size_t)kt * TK;
+#pragma unroll
+            for (int j = 0; j < X_PIECES; j++)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                             ::"s"(lds_address(x_dst + 8 * j * TK)), "v"(lane_off[j & 1]), "s"(src + (size_t)(8 * j) * K) : "memory");
+        } else {
+#pragma unroll
+            for (int j = 0; j < X_PIECES; j++) {
+                const int rr = min(8 * j + (lane >> 3), x_left - 1);
+                load16(x_dst + 8 * j * TK, x_share + (ptrdiff_t)rr * K + (size_t)kt * TK + 8 * lane_chunk[j & 1]);
             }
         }
     };
 
-    f32x4 acc[4][8];
+    f32x4 acc[4][NB];
 #pragma unroll
     for (int a = 0; a < 4; a++)
 #pragma unroll
-        for (int b = 0; b < 8; b++) acc[a][b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int b = 0; b < NB; b++) acc[a][b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    /* operand addresses inside a stage (elements): W rows n = 64 wn + 16 a + li, x rows m = 128 wm + 16 b + li;
+    /* operand addresses inside a stage (elements): W rows n = 64 wn + 16 a + li, x rows m = 16 NB wm + 16 b + li;
      * (row >> 1) & 7 = li >> 1 for both, whatever a or b */
     int a_rd[2], b_rd[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
         const int slot = 8 * ((4 * ks + lg) ^ (li >> 1));
         a_rd[ks] = (64 * wn + li) * TK + slot;
-        b_rd[ks] = DT * TK + (128 * wm + li) * TK + slot;
+        b_rd[ks] = TN * TK + (16 * NB * wm + li) * TK + slot;
     }
     const int nk = K / TK;
 
@@ -244,60 +304,61 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
     lds_barrier();
 
     for (int kt = 0; kt < nk; kt++) {
-        const uint16_t *cur = dlds + (kt & 1) * DSTAGE;
-        /* Four quarters per k tile: k-step ks, x blocks 4 half .. +3. The operands of the next quarter are
+        const uint16_t *cur = dlds + (kt & 1) * STAGE;
+        /* 2 HALVES steps per k tile: k-step ks, x blocks 4 half .. +3. The operands of the next step are
          * requested from LDS before the 16 MFMAs of this one are issued, so that the LDS works while the
-         * matrix core does; the W operands of a k-step are read with its first quarter. */
+         * matrix core does; the W operands of a k-step are read with its first step. */
         u32x4 av[2][4], bv[2][4];
-        auto read_quarter = [&](int qi) {
-            const int ks = qi >> 1, half = qi & 1;
+        auto read_step = [&](int step) {
+            const int ks = step / HALVES, half = step % HALVES;
             if (half == 0) {
 #pragma unroll
                 for (int a = 0; a < 4; a++) av[ks][a] = *reinterpret_cast<const u32x4 *>(&cur[a_rd[ks] + 16 * a * TK]);
             }
 #pragma unroll
-            for (int b = 0; b < 4; b++) bv[qi & 1][b] = *reinterpret_cast<const u32x4 *>(&cur[b_rd[ks] + 16 * (4 * half + b) * TK]);
+            for (int b = 0; b < 4; b++) bv[step & 1][b] = *reinterpret_cast<const u32x4 *>(&cur[b_rd[ks] + 16 * (4 * half + b) * TK]);
         };
-        read_quarter(0);
+        read_step(0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int qi = 0; qi < 4; qi++) {
-            if (qi < 3) read_quarter(qi + 1);
+        for (int step = 0; step < 2 * HALVES; step++) {
+            if (step + 1 < 2 * HALVES) read_step(step + 1);
             __builtin_amdgcn_sched_barrier(0);
-            const int ks = qi >> 1, half = qi & 1;
+            const int ks = step / HALVES, half = step % HALVES;
 #pragma unroll
             for (int a = 0; a < 4; a++)
 #pragma unroll
                 for (int b = 0; b < 4; b++)
                     acc[a][4 * half + b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        __builtin_bit_cast(bf16x8, av[ks][a]), __builtin_bit_cast(bf16x8, bv[qi & 1][b]), acc[a][4 * half + b], 0, 0, 0);
+                        __builtin_bit_cast(bf16x8, av[ks][a]), __builtin_bit_cast(bf16x8, bv[step & 1][b]), acc[a][4 * half + b], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             /* the next k tile: HBM/L2 -> the other stage, whose last readers passed the barrier that ended
-             * tile kt - 1. Requested behind the first quarter's MFMAs rather than right after the barrier,
+             * tile kt - 1. Requested behind the first step's MFMAs rather than right after the barrier,
              * where every wave would issue its requests before its first operand read. */
-            if (qi == 0 && kt + 1 < nk) { request(kt + 1, (kt + 1) & 1); __builtin_amdgcn_sched_barrier(0); }
+            if (step == 0 && kt + 1 < nk) { request(kt + 1, (kt + 1) & 1); __builtin_amdgcn_sched_barrier(0); }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       /* this wave's share of the next tile has landed */
         lds_barrier();                                          /* everybody's has, and nobody reads this tile any more */
     }
 
-    /* acc[a][b][r] = y[m0 + 128 wm + 16 b + li][n0 + 64 wn + 16 a + 4 lg + r].
+    /* acc[a][b][r] = y[m0 + 16 NB wm + 16 b + li][n0 + 64 wn + 16 a + 4 lg + r].
      * Stored straight from the accumulators a store instruction covers 16 rows x 64 (f32) or 32 (bf16) bytes,
-     * and the write path is bound by the number of such pieces, not by bytes. So the wave's 128 x 64 block
-     * goes through LDS (free after the loop's last barrier; 16 KB per wave, its own region, no workgroup
-     * barrier) and leaves as 16 B per lane along the rows: 4 rows x 256 B (f32) or 8 rows x 128 B (bf16) per
+     * and the write path is bound by the number of such pieces, not by bytes. So the wave's block goes
+     * through LDS (free after the loop's last barrier; 16 KB per wave, its own region, no workgroup barrier)
+     * and leaves as 16 B per lane along the rows: 4 rows x 256 B (f32) or 8 rows x 128 B (bf16) per
      * instruction. 16 B chunk c of row r sits in slot c ^ (r mod 16) (f32, 16 chunks a row) or
      * c ^ (r mod 8) (bf16, 8 chunks), which keeps both the writes and the reads off each other's banks.
      * LDS serves a wave's instructions in order, so the reads see the writes without a barrier. */
     constexpr int PER16 = 16 / (int)sizeof(OUT);               /* outputs per 16 B */
+    const int mw = m0 + 16 * NB * wm, nw = n0 + 64 * wn;
+    const float *bias = CONV ? geo.bias : nullptr;
     const bool staged = N % PER16 == 0 && ((uintptr_t)y & 15) == 0;
     if (staged) {
         uint16_t *mine = dlds + wave * 8192;                    /* 16 KB */
-        const int mw = m0 + 128 * wm, nw = n0 + 64 * wn;
         if constexpr (sizeof(OUT) == 4) {
-            float *buf = reinterpret_cast<float *>(mine);       /* 64 rows x 64 f32, half of the block at a time */
+            float *buf = reinterpret_cast<float *>(mine);       /* 64 rows x 64 f32 at a time */
 #pragma unroll
-            for (int half = 0; half < 2; half++) {
+            for (int half = 0; half < HALVES; half++) {
 #pragma unroll
                 for (int bb = 0; bb < 4; bb++)
 #pragma unroll
@@ -306,15 +367,18 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
 #pragma unroll
                 for (int it = 0; it < 16; it++) {
                     const int row = 4 * it + (lane >> 4), c = lane & 15;
-                    const f32x4 v = *reinterpret_cast<const f32x4 *>(&buf[row * 64 + 4 * (c ^ (row & 15))]);
+                    f32x4 v = *reinterpret_cast<const f32x4 *>(&buf[row * 64 + 4 * (c ^ (row & 15))]);
                     const int m = mw + 64 * half + row, n = nw + 4 * c;
-                    if (m < M && n < N) *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(y) + (size_t)m * N + n) = v;
+                    if (m < M && n < N) {
+                        if (bias) v += *reinterpret_cast<const f32x4 *>(bias + n);
+                        *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(y) + (size_t)m * N + n) = v;
+                    }
                 }
             }
         } else {
-            uint16_t *buf = mine;                               /* 128 rows x 64 bf16 */
+            uint16_t *buf = mine;                               /* 16 NB rows x 64 bf16 */
 #pragma unroll
-            for (int b = 0; b < 8; b++)
+            for (int b = 0; b < NB; b++)
 #pragma unroll
                 for (int a = 0; a < 4; a++) {
                     const int chunk = 2 * a + (lg >> 1);
@@ -322,7 +386,7 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
                         make_uint2(pack_bf16(acc[a][b][0], acc[a][b][1]), pack_bf16(acc[a][b][2], acc[a][b][3]));
                 }
 #pragma unroll
-            for (int it = 0; it < 16; it++) {
+            for (int it = 0; it < 2 * NB; it++) {
                 const int row = 8 * it + (lane >> 3), c = lane & 7;
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(&buf[row * 64 + 8 * (c ^ (row & 7))]);
                 const int m = mw + row, n = nw + 8 * c;
@@ -332,15 +396,37 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
         return;
     }
 #pragma unroll
-    for (int b = 0; b < 8; b++) {
-        const int m = m0 + 128 * wm + 16 * b + li;
+    for (int b = 0; b < NB; b++) {
+        const int m = mw + 16 * b + li;
         if (m >= M) continue;
 #pragma unroll
         for (int a = 0; a < 4; a++) {
-            const int n = n0 + 64 * wn + 16 * a + 4 * lg;
-            if (n < N) store4(y + (size_t)m * N + n, acc[a][b], N - n);
+            const int n = nw + 16 * a + 4 * lg;
+            if (n >= N) continue;
+            f32x4 v = acc[a][b];
+            if (bias)
+                for (int r = 0; r < 4 && n + r < N; r++) v[r] += bias[n + r];
+            store4(y + (size_t)m * N + n, v, N - n);
         }
     }
+}
+
+constexpr int DMA_LDS_BYTES = 128 * 1024;        /* two stages of (256 + 256) x 128 B; also the 8 x 16 KB of the epilogue */
+
+template <typename OUT, int TN, bool CONV>
+int launch_gemm_dma(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, int N, int K, const ConvGeom &geo) {
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_dma<OUT, TN, CONV>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, DMA_LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        configured = true;
+    }
+    const int tiles_m = (M + DT - 1) / DT, tiles_n = (N + TN - 1) / TN, total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    hipLaunchKernelGGL((k_gemm_dma<OUT, TN, CONV>), dim3((unsigned)per_xcd * 8), dim3(512), DMA_LDS_BYTES, st, y, x, W, M, N, K,
+                       tiles_m, total, per_xcd, geo);
+    return (int)hipGetLastError();
 }
 
 /* Any K / alignment: one thread per output element. */
@@ -362,19 +448,9 @@ int gemm(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, in
     if (M <= 0 || N <= 0) return 0;
     const bool aligned16 = ((uintptr_t)x & 15) == 0 && ((uintptr_t)W & 15) == 0;
     if (K > 0 && K % TK == 0 && aligned16 && M >= DT && N >= DT && (size_t)K * 2 * 8 < ((size_t)1 << 31)) {
-        static bool configured[2] = {false, false};
-        constexpr int which = sizeof(OUT) == 4 ? 0 : 1;
-        constexpr int lds_bytes = 2 * DSTAGE * (int)sizeof(uint16_t);
-        if (!configured[which]) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_dma<OUT>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-            if (e != hipSuccess) return (int)e;
-            configured[which] = true;
-        }
-        const int tiles_m = (M + DT - 1) / DT, tiles_n = (N + DT - 1) / DT, total = tiles_m * tiles_n;
-        const int per_xcd = (total + 7) / 8;
-        hipLaunchKernelGGL((k_gemm_dma<OUT>), dim3((unsigned)per_xcd * 8), dim3(512), lds_bytes, st, y, x, W, M, N, K,
-                           tiles_m, total, per_xcd);
+        const ConvGeom none = {};
+        const int e = launch_gemm_dma<OUT, 256, false>(st, y, x, W, M, N, K, none);
+        if (e) return e;
     } else if (K > 0 && K % 8 == 0 && aligned16) {
         /* 2 x 2 waves (128 x 128 tiles) measured best on the transformer shapes: 4 x 2 and 2 x 4 are
          * 5-8 % slower on the wide projections, 4 x 1 and 2 x 1 15-30 % slower. */
@@ -412,6 +488,11 @@ k_im2col(uint16_t *__restrict__ cols, const float *__restrict__ in, int h, int w
     }
 }
 
+__global__ void __launch_bounds__(64)
+k_zero_words(uint32_t *__restrict__ p, int n) {
+    for (int i = threadIdx.x; i < n; i += 64) p[i] = 0u;
+}
+
 __global__ void __launch_bounds__(256)
 k_add_bias_rows(float *__restrict__ y, const float *__restrict__ bias, int cols, size_t n) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -438,6 +519,40 @@ int iris_hip_conv2d(void *stream, uint16_t *scratch, size_t scratch_bytes, float
     const int ow = (width + pad_before + pad_after - k) / stride + 1;
     if (oh <= 0 || ow <= 0) return 0;
     const int ohw = oh * ow, row_len = k * k * cin;
+
+    /* Implicit GEMM: the image once as bf16 (the rows a chunk of output rows needs), then k_gemm_dma in its
+     * convolution mode straight on it; no patch matrix. Needs cin % 64 == 0 (a k tile inside one tap). */
+    const size_t in_row_bytes = (size_t)width * cin * sizeof(uint16_t), zero_bytes = 256;
+    if (cin % TK == 0 && cout >= 128 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)scratch & 15) == 0 &&
+        scratch_bytes > zero_bytes && (scratch_bytes - zero_bytes) / in_row_bytes >= (size_t)k) {
+        const long max_in_rows = (long)((scratch_bytes - zero_bytes) / in_row_bytes);
+        const long rows_out = (max_in_rows - k) / stride + 1;          /* (rows_out - 1) * stride + k <= max_in_rows */
+        hipLaunchKernelGGL(k_zero_words, dim3(1), dim3(64), 0, st, reinterpret_cast<uint32_t *>(scratch), (int)(zero_bytes / 4));
+        uint16_t *img = scratch + zero_bytes / sizeof(uint16_t);
+        const bool bias_fused = bias && ((uintptr_t)bias & 15) == 0;
+        for (long r0 = 0; r0 < oh; r0 += rows_out) {
+            const long r1 = r0 + rows_out < oh ? r0 + rows_out : oh;
+            const long y_lo = r0 * stride - pad_before > 0 ? r0 * stride - pad_before : 0;
+            const long y_hi = (r1 - 1) * stride - pad_before + k < h ? (r1 - 1) * stride - pad_before + k : h;
+            if (y_hi > y_lo) {
+                int e = iris_hip_f32_to_bf16(stream, img, in + (size_t)y_lo * width * cin, (size_t)(y_hi - y_lo) * width * cin);
+                if (e) return e;
+            }
+            const ConvGeom geo = {h, width, cin, k, stride, pad_before, ow, (int)(r0 * ow), scratch, bias_fused ? bias : nullptr};
+            const uint16_t *virtual_image = img - (size_t)y_lo * width * cin;     /* row y of the image at + y * width * cin */
+            float *dst = out + (size_t)r0 * ow * cout;
+            const int m = (int)((r1 - r0) * ow);
+            const int e = cout >= 256 ? launch_gemm_dma<float, 256, true>(st, dst, virtual_image, w, m, cout, row_len, geo)
+                                      : launch_gemm_dma<float, 128, true>(st, dst, virtual_image, w, m, cout, row_len, geo);
+            if (e) return e;
+        }
+        if (bias && !bias_fused) {
+            const size_t n = (size_t)ohw * cout;
+            hipLaunchKernelGGL(k_add_bias_rows, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, out, bias, cout, n);
+        }
+        return (int)hipGetLastError();
+    }
+
     long chunk = (long)(scratch_bytes / ((size_t)row_len * sizeof(uint16_t)));
     if (chunk < 1) return (int)hipErrorInvalidValue;
     if (chunk > ohw) chunk = ohw;

@@ -182,7 +182,12 @@ def test_swiglu(dev, orc, rows, cols, ldi, ldo):
 
 # ------------------------------------------------------------------ VAE layers
 @pytest.mark.parametrize("h,w,cin,cout,k,stride,pb,pa", [(6, 5, 8, 4, 3, 1, 1, 1), (7, 7, 3, 5, 3, 1, 1, 1), (8, 8, 16, 6, 3, 2, 0, 1),
-                                                         (16, 16, 128, 128, 3, 1, 1, 1), (9, 9, 32, 64, 1, 1, 0, 0)])
+                                                         (16, 16, 128, 128, 3, 1, 1, 1), (9, 9, 32, 64, 1, 1, 0, 0),
+                                                         # cin % 64 == 0 and cout >= 128: the implicit-GEMM path
+                                                         (20, 17, 64, 128, 3, 1, 1, 1), (16, 16, 128, 256, 3, 1, 1, 1),
+                                                         (33, 20, 64, 320, 3, 2, 0, 1), (12, 12, 128, 130, 1, 1, 0, 0),
+                                                         (24, 40, 192, 128, 3, 1, 1, 1), (5, 4, 64, 512, 3, 1, 1, 1),
+                                                         (40, 36, 128, 128, 3, 2, 1, 1)])
 def test_conv2d(dev, orc, h, w, cin, cout, k, stride, pb, pa):
     img = rnd((h * w, cin), h + cin)
     wt = O.f32_to_bf16(rnd((cout, k * k * cin), cout, 0.1))
@@ -197,6 +202,36 @@ def test_conv2d(dev, orc, h, w, cin, cout, k, stride, pb, pa):
     dout = dev.alloc(want.size * 4)
     got = run(dev, lambda: dev.lib.iris_dev_conv2d(dout, dimg, dw, None, h, w, cin, cout, k, stride, pb, pa), [(dout, want.shape, np.float32)])
     np.testing.assert_allclose(got, want - bias[None, :], atol=2e-5 * np.sqrt(k * k * cin))
+
+
+def test_conv2d_large_image_in_chunks_sampled_pixels(dev):
+    """An image whose bf16 copy does not fit the library's 256 MB of convolution scratch is processed in
+    chunks of output rows with their halo rows. 1040 x 1024 x 128 -> 128, 3 x 3: sampled output pixels
+    (corners, edges, the rows around every possible chunk boundary, random ones) against the definition
+    in float64 on bf16-rounded inputs."""
+    h, w, cin, cout, k = 1040, 1024, 128, 128, 3
+    rng = np.random.default_rng(11)
+    img = rng.standard_normal((h * w, cin), dtype=np.float32)
+    wt = O.f32_to_bf16((rng.standard_normal((cout, k * k * cin)) * 0.05).astype(np.float32))
+    bias = rng.standard_normal(cout).astype(np.float32)
+    dimg, dw, db = dev.put(img), dev.put(wt), dev.put(bias)
+    dout = dev.alloc(h * w * cout * 4)
+    got = run(dev, lambda: dev.lib.iris_dev_conv2d(dout, dimg, dw, db, h, w, cin, cout, k, 1, 1, 1), [(dout, (h * w, cout), np.float32)])
+    wf = O.bf16_to_f32(wt).astype(np.float64).reshape(cout, k, k, cin)
+    ys = np.r_[0, 1, h - 2, h - 1, rng.integers(0, h, 40), np.arange(1016, 1030)]
+    xs = np.r_[0, 1, w - 2, w - 1, rng.integers(0, w, 12)]
+    image = img.reshape(h, w, cin)
+    worst = 0.0
+    for yy in ys:
+        for xx in xs:
+            acc = bias.astype(np.float64).copy()
+            for ky in range(k):
+                for kx in range(k):
+                    iy, ix = yy + ky - 1, xx + kx - 1
+                    if 0 <= iy < h and 0 <= ix < w:
+                        acc += wf[:, ky, kx, :] @ O.bf16_to_f32(O.f32_to_bf16(image[iy, ix])).astype(np.float64)
+            worst = max(worst, float(np.abs(got[yy * w + xx] - acc).max()))
+    assert worst <= 2e-5 * np.sqrt(k * k * cin) * 4, worst
 
 
 @pytest.mark.parametrize("hw,c,groups,silu", [(30, 16, 4, 0), (4096, 128, 32, 1), (100, 6, 3, 1)])
