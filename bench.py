@@ -263,6 +263,21 @@ def other_ops(dev, hip, stream, rng, settle_ms=0.0):
                     "gbps": round(nbytes / ms / 1e6, 0)})
     for p in (x, W, y, w1):
         lib.iris_dev_free(p)
+    # the VAE's operators at two of its shapes: 3 x 3 convolution and group norm + SiLU, channels last, f32 in and out
+    for side, ch in ((512, 128), (256, 512)):
+        hw = side * side
+        img = dev.to_device(rng.standard_normal((hw, ch), dtype=np.float32))
+        out = lib.iris_dev_alloc(hw * ch * 4)
+        wt = dev.to_device(to_bf16(rng.standard_normal((ch, 9 * ch), dtype=np.float32) * 0.02))
+        g1 = dev.to_device(np.ones(ch, np.float32))
+        ms = timed(lambda i: lib.iris_dev_conv2d(out, img, wt, g1, side, side, ch, ch, 3, 1, 1, 1), 5)
+        res.append({"op": "conv2d 3x3", "shape": f"{side}x{side}x{ch}->{ch}", "us": round(ms * 1e3, 1),
+                    "tflops": round(2 * hw * 9 * ch * ch / ms / 1e9, 1)})
+        ms = timed(lambda i: lib.iris_dev_group_norm(out, img, g1, g1, hw, ch, 32, 1e-6, 1), 5)
+        res.append({"op": "group_norm+silu", "shape": f"{side}x{side}x{ch}", "us": round(ms * 1e3, 1),
+                    "gbps": round(8 * hw * ch / ms / 1e6, 0)})
+        for p in (img, out, wt, g1):
+            lib.iris_dev_free(p)
     return res
 
 
