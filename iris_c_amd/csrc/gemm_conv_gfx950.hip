@@ -199,10 +199,17 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
     constexpr int W_PIECES = TN / 64, X_PIECES = 4;            /* 8-row pieces per wave and k tile */
     constexpr int STAGE = (TN + DT) * TK;                      /* elements: W tile then x tile */
     extern __shared__ __align__(16) uint16_t dlds[];          /* two stages (and room for the epilogue) */
-    /* each XCD (own L2) walks a contiguous range of the tile list, m fastest: neighbours share a W tile */
+    /* Each XCD (own L2) walks a contiguous range of the tile list. The list runs through bands of 8 tile rows
+     * (m), inside a band m fastest and then n: the 32 workgroups an XCD runs at a time then form an 8 x 4
+     * block of tiles that needs 8 x tiles and 4 W tiles per k step, where a whole column of tile rows at a
+     * time would need all of x again for every column of W. */
     const int work = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (work >= total) return;
-    const int bm = work % tiles_m, bn = work / tiles_m;
+    constexpr int BAND = 8;
+    const int tiles_n = total / tiles_m;
+    const int band = work / (BAND * tiles_n), in_band = work - band * (BAND * tiles_n);
+    const int band_rows = min(tiles_m - band * BAND, BAND);
+    const int bm = band * BAND + in_band % band_rows, bn = in_band / band_rows;
     const int m0 = bm * DT, n0 = bn * TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
