@@ -473,6 +473,13 @@ def main():
     res = Resident(dev, c2, copies)
     flops = attention_flops(c2)
 
+    # for the record: the same step timed right after the GPU sat idle during the uploads, clocks not yet settled
+    lib.iris_dev_sync()
+    t0 = time.perf_counter()
+    for i in range(50):
+        res.step(i)
+    lib.iris_dev_sync()
+    idle_ms = (time.perf_counter() - t0) / 50 * 1e3
     settle_steps = settle(lib, res.step, args.settle_ms)
     for i in range(args.warmup):
         res.step(i)
@@ -522,6 +529,9 @@ def main():
         "config": {"workload": "C2: norm+rope(Q), norm+rope(K), joint attention; 24 heads x 128, 512 text + 4096 image "
                                "tokens, fused qkv rows (ldi 9216), one sequence",
                    "device": dev.name()},
+        "first_50_steps_after_idle": {"ms_per_step": round(idle_ms, 4), "tflops": round(flops / (idle_ms * 1e-3) / 1e12, 2),
+                                      "note": "before the settling load: the clocks take tens of ms of load to reach their "
+                                              "steady state (includes first-launch costs)"},
         "step_with_fused_qk_norm": None if fused_ms is None else {
             "ms_per_step": round(fused_ms, 4), "tflops": round(flops / (fused_ms * 1e-3) / 1e12, 2),
             "note": "two launches: iris_dev_head_norm_rope_qk + iris_dev_attention"},
