@@ -1,4 +1,9 @@
-"""One single-stream transformer block issued the way the reference issues it
+"""Whole blocks of the models, issued the way the reference issues them, against
+the same chains composed from the CPU oracle's operators: a FLUX
+single-stream block, a text-encoder layer and the VAE's residual and
+attention blocks.
+
+The single-stream transformer block
 (iris_transformer_flux.c:3826-3839): layer norm + modulation, the fused
 input projection into [q | k | v | gate | up] rows, norm+rope on the Q and K
 columns of those rows, joint attention writing into the first columns of the
@@ -94,3 +99,127 @@ def test_single_stream_block_chain(dev, orc, seq, heads, mlp, backend):
     mx, mean = error_stats(got - b["x"], want - b["x"])
     assert mx <= 3e-2 and mean <= 3e-3, f"max-abs {mx:.4g}, mean-abs {mean:.4g}"
     assert np.array_equal(got, fused), "the block with Q normalised inside attention differs from the three-call block"
+
+
+# ------------------------------------------------------------------ text encoder layer (iris_qwen3.c:1586-1604)
+def test_text_encoder_layer_chain(dev, orc):
+    """RMS norm, fused q | k | v projection with 8 query heads on 2 kv heads, split-half norm+rope on the Q and
+    K columns, causal attention with a right-padding mask, output projection, plain residual, SwiGLU MLP."""
+    rng = np.random.default_rng(21)
+    seq, length, heads, kv, hidden, inter = 200, 137, 8, 2, 640, 1280
+    q_dim, kv_dim = heads * 128, kv * 128
+    ld = q_dim + 2 * kv_dim
+    f = lambda *shape, s=1.0: (rng.standard_normal(shape) * s).astype(np.float32)
+    x0 = f(seq, hidden, s=1.5)
+    in_norm, post_norm = 1 + f(hidden, s=0.05), 1 + f(hidden, s=0.05)
+    w_qkv, w_o = O.f32_to_bf16(f(ld, hidden, s=1 / np.sqrt(hidden))), O.f32_to_bf16(f(hidden, q_dim, s=1 / np.sqrt(q_dim)))
+    w_gu, w_down = O.f32_to_bf16(f(2 * inter, hidden, s=1 / np.sqrt(hidden))), O.f32_to_bf16(f(hidden, inter, s=1 / np.sqrt(inter)))
+    q_norm, k_norm = 1 + f(128, s=0.05), 1 + f(128, s=0.05)
+    mask = (np.arange(seq) < length).astype(np.int32)
+    cos, sin = orc.qwen3_rope_table(seq, 128, 1e6, mask=mask)
+    scale, eps = float(1 / np.sqrt(128.0)), 1e-6
+
+    # oracle chain
+    norm = orc.dev_rms_norm_mod(x0, in_norm, None, eps)
+    qkv = O.f32_to_bf16(orc.dev_linear(norm, w_qkv))
+    orc.head_norm_rope_bf16(qkv, ld, q_norm, cos, sin, seq, heads, 128, eps, 1, col0=0)
+    orc.head_norm_rope_bf16(qkv, ld, k_norm, cos, sin, seq, kv, 128, eps, 1, col0=q_dim)
+    att = O.f32_to_bf16(orc.attention_bf16(qkv, ld, 0, q_dim, q_dim + kv_dim, seq, seq, heads, kv, 128, scale, True, mask))
+    x1 = orc.dev_residual(x0, orc.dev_linear(att, w_o), None)
+    norm2 = orc.dev_rms_norm_mod(x1, post_norm, None, eps)
+    gate_up = O.f32_to_bf16(orc.dev_linear(norm2, w_gu))
+    act = orc.dev_swiglu(gate_up, inter)
+    want = orc.dev_residual(x1, orc.dev_linear(act, w_down), None)
+
+    # device chain
+    lib = dev.lib
+    d = {k: dev.put(v) for k, v in dict(x=x0, in_norm=in_norm, post_norm=post_norm, w_qkv=w_qkv, w_o=w_o, w_gu=w_gu, w_down=w_down,
+                                        q_norm=q_norm, k_norm=k_norm, cos=cos, sin=sin, mask=mask).items()}
+    normb, qkvb, attb = dev.alloc(seq * hidden * 2), dev.alloc(seq * ld * 2), dev.alloc(seq * q_dim * 2)
+    outb, gub, actb = dev.alloc(seq * hidden * 4), dev.alloc(seq * 2 * inter * 2), dev.alloc(seq * inter * 2)
+    col = lambda p, elems: ptr_add(p, 2 * elems)
+    lib.iris_dev_rms_norm(normb, d["x"], d["in_norm"], seq, hidden, eps)
+    lib.iris_dev_linear_bf16(qkvb, normb, d["w_qkv"], seq, hidden, ld)
+    lib.iris_dev_head_norm_rope(qkvb, ld, d["q_norm"], d["cos"], d["sin"], seq, heads, 128, eps, 1)
+    lib.iris_dev_head_norm_rope(col(qkvb, q_dim), ld, d["k_norm"], d["cos"], d["sin"], seq, kv, 128, eps, 1)
+    lib.iris_dev_attention(attb, q_dim, qkvb, col(qkvb, q_dim), col(qkvb, q_dim + kv_dim), ld, seq, seq, heads, kv, 128, scale, 1,
+                           d["mask"])
+    assert dev.dev.last_kernel() == "fa_hd128"
+    lib.iris_dev_linear_f32(outb, attb, d["w_o"], seq, q_dim, hidden)
+    lib.iris_dev_residual(d["x"], outb, None, seq, hidden)
+    lib.iris_dev_rms_norm(normb, d["x"], d["post_norm"], seq, hidden, eps)
+    lib.iris_dev_linear_bf16(gub, normb, d["w_gu"], seq, hidden, 2 * inter)
+    lib.iris_dev_swiglu(actb, inter, gub, col(gub, inter), 2 * inter, seq, inter)
+    lib.iris_dev_linear_f32(outb, actb, d["w_down"], seq, inter, hidden)
+    lib.iris_dev_residual(d["x"], outb, None, seq, hidden)
+    dev.check()
+    got = dev.get(d["x"], (seq, hidden), np.float32)
+    dev.free_all()
+    mx, mean = error_stats(got - x0, want - x0)
+    assert mx <= 5e-2 and mean <= 4e-3, f"max-abs {mx:.4g}, mean-abs {mean:.4g}"
+
+
+# ------------------------------------------------------------------ VAE residual block and attention (iris_vae.c:1095-1127)
+def test_vae_resblock_and_attention_chain(dev, orc):
+    """out = x + conv2(silu(gn2(conv1(silu(gn1(x)))))) with a 1 x 1 convolution on the skip path (256 -> 128
+    channels), then the single-head self-attention over the pixels as the reference issues it: group norm, q | k | v
+    as a 1 x 1 convolution over an (hw x 1) image, conversion to bf16, attention with head_dim = channels, output
+    projection, bias, residual."""
+    rng = np.random.default_rng(31)
+    h, w, cin, cout, groups, eps = 12, 10, 256, 128, 32, 1e-6
+    hw = h * w
+    f = lambda *shape, s=1.0: (rng.standard_normal(shape) * s).astype(np.float32)
+    x = f(hw, cin)
+    n1w, n1b, n2w, n2b = 1 + f(cin, s=0.1), f(cin, s=0.1), 1 + f(cout, s=0.1), f(cout, s=0.1)
+    c1w, c1b = O.f32_to_bf16(f(cout, 9 * cin, s=1 / np.sqrt(9 * cin))), f(cout, s=0.1)
+    c2w, c2b = O.f32_to_bf16(f(cout, 9 * cout, s=1 / np.sqrt(9 * cout))), f(cout, s=0.1)
+    skw, skb = O.f32_to_bf16(f(cout, cin, s=1 / np.sqrt(cin))), f(cout, s=0.1)
+    # attention over `cout` = 128 channels here would take the 128-wide kernel; the VAE's is 512 wide: its own tensors
+    c = 512
+    xa = f(hw, c)
+    anw, anb = 1 + f(c, s=0.1), f(c, s=0.1)
+    qkvw, qkvb = O.f32_to_bf16(f(3 * c, c, s=1 / np.sqrt(c))), f(3 * c, s=0.1)
+    ow_, ob_ = O.f32_to_bf16(f(c, c, s=1 / np.sqrt(c))), f(c, s=0.1)
+
+    # oracle
+    t1 = orc.dev_group_norm(x, n1w, n1b, groups, eps, 1)
+    t2 = orc.dev_conv2d(t1, c1w, c1b, h, w, 3, 1, 1, 1)
+    t1 = orc.dev_group_norm(t2, n2w, n2b, groups, eps, 1)
+    out = orc.dev_conv2d(t1, c2w, c2b, h, w, 3, 1, 1, 1)
+    want_res = orc.dev_add(out, orc.dev_conv2d(x, skw, skb, h, w, 1, 1, 0, 0))
+    g = orc.dev_group_norm(xa, anw, anb, groups, eps, 0)
+    qkv = O.f32_to_bf16(orc.dev_conv2d(g, qkvw, qkvb, hw, 1, 1, 1, 0, 0))
+    o = O.f32_to_bf16(orc.attention_bf16(qkv, 3 * c, 0, c, 2 * c, hw, hw, 1, 1, c, float(1 / np.sqrt(c))))
+    want_att = orc.dev_add(orc.dev_add_bias(orc.dev_linear(o, ow_), ob_), xa)
+
+    # device
+    lib = dev.lib
+    d = {k: dev.put(v) for k, v in dict(x=x, n1w=n1w, n1b=n1b, n2w=n2w, n2b=n2b, c1w=c1w, c1b=c1b, c2w=c2w, c2b=c2b, skw=skw, skb=skb,
+                                        xa=xa, anw=anw, anb=anb, qkvw=qkvw, qkvb=qkvb, ow=ow_, ob=ob_).items()}
+    big = hw * max(cin, 3 * c) * 4
+    t1b, t2b, outb = dev.alloc(big), dev.alloc(big), dev.alloc(big)
+    lib.iris_dev_group_norm(t1b, d["x"], d["n1w"], d["n1b"], hw, cin, groups, eps, 1)
+    lib.iris_dev_conv2d(t2b, t1b, d["c1w"], d["c1b"], h, w, cin, cout, 3, 1, 1, 1)
+    lib.iris_dev_group_norm(t1b, t2b, d["n2w"], d["n2b"], hw, cout, groups, eps, 1)
+    lib.iris_dev_conv2d(outb, t1b, d["c2w"], d["c2b"], h, w, cout, cout, 3, 1, 1, 1)
+    lib.iris_dev_conv2d(t2b, d["x"], d["skw"], d["skb"], h, w, cin, cout, 1, 1, 0, 0)
+    lib.iris_dev_add(outb, t2b, hw * cout)
+    dev.check()
+    got_res = dev.get(outb, (hw, cout), np.float32)
+    qkvd = dev.alloc(hw * 4 * c * 2)
+    od = ptr_add(qkvd, 2 * hw * 3 * c)
+    lib.iris_dev_group_norm(t1b, d["xa"], d["anw"], d["anb"], hw, c, groups, eps, 0)
+    lib.iris_dev_conv2d(t2b, t1b, d["qkvw"], d["qkvb"], hw, 1, c, 3 * c, 1, 1, 0, 0)
+    lib.iris_dev_f32_to_bf16(qkvd, t2b, hw * 3 * c)
+    lib.iris_dev_attention(od, c, qkvd, ptr_add(qkvd, 2 * c), ptr_add(qkvd, 4 * c), 3 * c, hw, hw, 1, 1, c, float(1 / np.sqrt(c)), 0, None)
+    assert dev.dev.last_kernel() == "fa_sliced"
+    lib.iris_dev_linear_f32(outb, od, d["ow"], hw, c, c)
+    lib.iris_dev_add_bias(outb, d["ob"], hw, c)
+    lib.iris_dev_add(outb, d["xa"], hw * c)
+    dev.check()
+    got_att = dev.get(outb, (hw, c), np.float32)
+    dev.free_all()
+    mx, mean = error_stats(got_res, want_res)
+    assert mx <= 3e-2 and mean <= 3e-3, f"resblock: max-abs {mx:.4g}, mean-abs {mean:.4g}"
+    mx, mean = error_stats(got_att - xa, want_att - xa)
+    assert mx <= 3e-2 and mean <= 3e-3, f"attention block: max-abs {mx:.4g}, mean-abs {mean:.4g}"
