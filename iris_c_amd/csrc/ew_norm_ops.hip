@@ -345,33 +345,48 @@ k_gn_moments_any(Moments *__restrict__ part, const float *__restrict__ in, int h
     if (threadIdx.x == 0) part[(size_t)g * gridDim.y + b] = sh[0];
 }
 
-/* stats[g] = mean, stats[groups + g] = 1 / sqrt(var + eps): the partial moments merged in double, one
- * wave per group (each lane merges its share of the workgroups' partials, then the lanes merge pairwise) */
-__device__ __forceinline__ void merge64(double &n, double &mean, double &m2, double nb, double mb, double m2b) {
-    if (nb == 0.0) return;
-    const double tot = n + nb, d = mb - mean;
-    mean += d * (nb / tot);
-    m2 += m2b + d * d * (n * nb / tot);
-    n = tot;
+/* stats[g] = mean, stats[groups + g] = 1 / sqrt(var + eps) from the workgroups' partial moments, in double, one
+ * workgroup per group: the mean is the count-weighted mean of the partial means, the sum of squared deviations is
+ * the sum of the partial ones plus count x (partial mean - mean)^2 -- the same combination as the pairwise
+ * merge, written so that it takes two sums over the partials and a single division. */
+__device__ __forceinline__ double wave_sum64(double v) {
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
 }
 
-__global__ void __launch_bounds__(64)
+/* one workgroup of 256 threads per group; a thread holds up to GN_MAX_BLOCKS / 256 partials, loaded together */
+__device__ __forceinline__ double block_sum64(double v, double *sh) {
+    v = wave_sum64(v);
+    __syncthreads();                                   /* sh may still be read from the previous call */
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (sh[0] + sh[1]) + (sh[2] + sh[3]);
+}
+
+__global__ void __launch_bounds__(256)
 k_gn_finish(float *__restrict__ stats, const Moments *__restrict__ part, int groups, int nblocks, float eps) {
-    const int g = blockIdx.x, lane = threadIdx.x;
-    double n = 0.0, mean = 0.0, m2 = 0.0;
-    for (int b = lane; b < nblocks; b += 64) {
-        const Moments m = part[(size_t)g * nblocks + b];
-        merge64(n, mean, m2, (double)m.n, (double)m.mean, (double)m.m2);
+    __shared__ double sh[4];
+    constexpr int PER = GN_MAX_BLOCKS / 256;
+    const int g = blockIdx.x;
+    Moments m[PER];
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int b = threadIdx.x + 256 * i;
+        m[i] = b < nblocks ? part[(size_t)g * nblocks + b] : Moments{0.0f, 0.0f, 0.0f};
     }
-    for (int off = 32; off > 0; off >>= 1) {
-        const double nb = __shfl_xor(n, off, 64), mb = __shfl_xor(mean, off, 64), m2b = __shfl_xor(m2, off, 64);
-        /* both partners must end with the same value: merge in a fixed order (lower lane first) */
-        double n0 = n, mean0 = mean, m20 = m2, n1 = nb, mean1 = mb, m21 = m2b;
-        if (lane & off) { n0 = nb; mean0 = mb; m20 = m2b; n1 = n; mean1 = mean; m21 = m2; }
-        merge64(n0, mean0, m20, n1, mean1, m21);
-        n = n0; mean = mean0; m2 = m20;
+    double n = 0.0, weighted = 0.0;
+#pragma unroll
+    for (int i = 0; i < PER; i++) { n += (double)m[i].n; weighted += (double)m[i].n * (double)m[i].mean; }
+    n = block_sum64(n, sh);
+    const double mean = n > 0.0 ? block_sum64(weighted, sh) / n : 0.0;
+    double m2 = 0.0;
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const double d = (double)m[i].mean - mean;
+        m2 += (double)m[i].m2 + (double)m[i].n * d * d;
     }
-    if (lane == 0) {
+    m2 = block_sum64(m2, sh);
+    if (threadIdx.x == 0) {
         stats[g] = (float)mean;
         stats[groups + g] = (float)(1.0 / sqrt((n > 0.0 ? m2 / n : 0.0) + (double)eps));
     }
@@ -499,7 +514,7 @@ int iris_hip_group_norm(void *stream, float *scratch, float *out, const float *i
         if (nblocks > GN_MAX_BLOCKS) nblocks = GN_MAX_BLOCKS;
         hipLaunchKernelGGL(k_gn_moments_any, dim3(groups, nblocks), dim3(ROW_THREADS), 0, st, part, in, hw, c, cg);
     }
-    hipLaunchKernelGGL(k_gn_finish, dim3(groups), dim3(64), 0, st, stats, part, groups, nblocks, eps);
+    hipLaunchKernelGGL(k_gn_finish, dim3(groups), dim3(256), 0, st, stats, part, groups, nblocks, eps);
     const size_t n = (size_t)hw * c;
     if (al16(out) && al16(in) && al16(gamma) && al16(beta) && c % 4 == 0)
         hipLaunchKernelGGL(k_gn_normalize<4>, dim3(blocks_for(n, EW_THREADS * 4)), dim3(EW_THREADS), 0, st, out, in, stats, gamma, beta, c, cg, groups, do_silu, n);

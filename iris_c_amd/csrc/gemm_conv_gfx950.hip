@@ -517,7 +517,16 @@ int iris_hip_linear_bf16(void *stream, uint16_t *y, const uint16_t *x, const uin
     return gemm<uint16_t>((hipStream_t)stream, y, x, W, rows, out, in);
 }
 
-/* scratch: device buffer of scratch_bytes (>= one patch row) for the bf16 patches */
+/* Zeroes the first IRIS_CONV_ZERO_BYTES of a freshly allocated convolution scratch buffer: the page that taps
+ * outside the image read. iris_hip_conv2d never writes there. */
+int iris_hip_conv2d_prepare_scratch(void *stream, uint16_t *scratch) {
+    hipLaunchKernelGGL(k_zero_words, dim3(1), dim3(64), 0, (hipStream_t)stream, reinterpret_cast<uint32_t *>(scratch),
+                       IRIS_CONV_ZERO_BYTES / 4);
+    return (int)hipGetLastError();
+}
+
+/* scratch: device buffer of scratch_bytes, 16-byte aligned, prepared once by iris_hip_conv2d_prepare_scratch: the
+ * page of zeros, then room for the bf16 image rows of a chunk or (gathered shapes) at least one patch row */
 int iris_hip_conv2d(void *stream, uint16_t *scratch, size_t scratch_bytes, float *out, const float *in,
                     const uint16_t *w, const float *bias, int h, int width, int cin, int cout, int k,
                     int stride, int pad_before, int pad_after) {
@@ -529,13 +538,16 @@ int iris_hip_conv2d(void *stream, uint16_t *scratch, size_t scratch_bytes, float
 
     /* Implicit GEMM: the image once as bf16 (the rows a chunk of output rows needs), then k_gemm_dma in its
      * convolution mode straight on it; no patch matrix. Needs cin % 64 == 0 (a k tile inside one tap). */
-    const size_t in_row_bytes = (size_t)width * cin * sizeof(uint16_t), zero_bytes = 256;
+    if (scratch_bytes <= IRIS_CONV_ZERO_BYTES) return (int)hipErrorInvalidValue;
+    const uint16_t *zeros = scratch;
+    scratch += IRIS_CONV_ZERO_BYTES / sizeof(uint16_t);
+    scratch_bytes -= IRIS_CONV_ZERO_BYTES;
+    const size_t in_row_bytes = (size_t)width * cin * sizeof(uint16_t);
     if (cin % TK == 0 && cout >= 128 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)scratch & 15) == 0 &&
-        scratch_bytes > zero_bytes && (scratch_bytes - zero_bytes) / in_row_bytes >= (size_t)k) {
-        const long max_in_rows = (long)((scratch_bytes - zero_bytes) / in_row_bytes);
+        scratch_bytes / in_row_bytes >= (size_t)k) {
+        const long max_in_rows = (long)(scratch_bytes / in_row_bytes);
         const long rows_out = (max_in_rows - k) / stride + 1;          /* (rows_out - 1) * stride + k <= max_in_rows */
-        hipLaunchKernelGGL(k_zero_words, dim3(1), dim3(64), 0, st, reinterpret_cast<uint32_t *>(scratch), (int)(zero_bytes / 4));
-        uint16_t *img = scratch + zero_bytes / sizeof(uint16_t);
+        uint16_t *img = scratch;
         const bool bias_fused = bias && ((uintptr_t)bias & 15) == 0;
         for (long r0 = 0; r0 < oh; r0 += rows_out) {
             const long r1 = r0 + rows_out < oh ? r0 + rows_out : oh;
@@ -545,7 +557,7 @@ int iris_hip_conv2d(void *stream, uint16_t *scratch, size_t scratch_bytes, float
                 int e = iris_hip_f32_to_bf16(stream, img, in + (size_t)y_lo * width * cin, (size_t)(y_hi - y_lo) * width * cin);
                 if (e) return e;
             }
-            const ConvGeom geo = {h, width, cin, k, stride, pad_before, ow, (int)(r0 * ow), scratch, bias_fused ? bias : nullptr};
+            const ConvGeom geo = {h, width, cin, k, stride, pad_before, ow, (int)(r0 * ow), zeros, bias_fused ? bias : nullptr};
             const uint16_t *virtual_image = img - (size_t)y_lo * width * cin;     /* row y of the image at + y * width * cin */
             float *dst = out + (size_t)r0 * ow * cout;
             const int m = (int)((r1 - r0) * ow);

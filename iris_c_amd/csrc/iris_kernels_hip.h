@@ -87,7 +87,11 @@ int iris_hip_group_norm(void *stream, float *scratch, float *out, const float *i
  * x, W are 16-byte aligned, scalar kernel otherwise */
 int iris_hip_linear_f32(void *stream, float *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out);
 int iris_hip_linear_bf16(void *stream, uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out);
-/* convolution through bf16 patches in `scratch` (scratch_bytes >= 2 * k * k * cin) */
+/* Convolution. `scratch` is a private device buffer, 16-byte aligned, whose first IRIS_CONV_ZERO_BYTES are zeroed
+ * once by iris_hip_conv2d_prepare_scratch and never written again (the page that taps outside the image read);
+ * the rest holds the image as bf16 (or the bf16 patches of the shapes that are gathered: >= 2 * k * k * cin bytes). */
+#define IRIS_CONV_ZERO_BYTES 256
+int iris_hip_conv2d_prepare_scratch(void *stream, uint16_t *scratch);
 int iris_hip_conv2d(void *stream, uint16_t *scratch, size_t scratch_bytes, float *out, const float *in,
                     const uint16_t *w, const float *bias, int h, int width, int cin, int cout, int k,
                     int stride, int pad_before, int pad_after);

@@ -379,15 +379,19 @@ void iris_dev_conv2d(float *out, const float *in, const uint16_t *w, const float
                      int pad_before, int pad_after) {
     if (!need_ready("conv2d")) return;
     if (h <= 0 || width <= 0 || cin <= 0 || cout <= 0 || k <= 0 || stride <= 0 || pad_before < 0 || pad_after < 0 ||
-        (size_t)k * k * cin * sizeof(uint16_t) > CONV_SCRATCH_BYTES) {
+        (size_t)k * k * cin * sizeof(uint16_t) > CONV_SCRATCH_BYTES - IRIS_CONV_ZERO_BYTES) {
         fail(-1, "conv2d", "bad shape");
         return;
     }
-    if (!g_conv_scratch && hipMalloc((void **)&g_conv_scratch, CONV_SCRATCH_BYTES) != hipSuccess) {
-        (void)hipGetLastError();
-        g_conv_scratch = NULL;
-        fail(-1, "conv2d", "scratch allocation failed");
-        return;
+    if (!g_conv_scratch) {
+        if (hipMalloc((void **)&g_conv_scratch, CONV_SCRATCH_BYTES) != hipSuccess) {
+            (void)hipGetLastError();
+            g_conv_scratch = NULL;
+            fail(-1, "conv2d", "scratch allocation failed");
+            return;
+        }
+        int e = iris_hip_conv2d_prepare_scratch(g_stream, g_conv_scratch);
+        if (e) { check((hipError_t)e, "conv2d scratch"); return; }
     }
     int err = iris_hip_conv2d(g_stream, g_conv_scratch, CONV_SCRATCH_BYTES, out, in, w, bias, h, width, cin, cout,
                               k, stride, pad_before, pad_after);
