@@ -8,13 +8,15 @@
  *   iris_rope_*      host builders, plain C + libm, bit-identical to the
  *                    reference's routines (same float / double arithmetic,
  *                    same libm calls on the same arguments);
- *   iris_dev_rope_*  the same tables written straight into device memory by a
- *                    kernel: the host only lays out the integer (or
- *                    half-integer) positions, 16 bytes a row instead of 512,
- *                    and no cosf/sinf runs on the host. Angles are formed by
- *                    the same float (or double) multiply as on the host and
- *                    the cosine and sine are evaluated in double, so every
- *                    entry is within 1 float ulp of the host table.
+ *   iris_dev_rope_*  the same tables written straight into device memory, with the
+ *                    same bits: the host evaluates each DISTINCT (axis,
+ *                    position) of the sequence once, with those same libm
+ *                    calls (an h x w image has h + w distinct positions per
+ *                    axis, not h * w), uploads that dictionary plus one
+ *                    32-bit offset per (token, axis) -- 16 bytes a token for
+ *                    four axes instead of the 512 bytes of its two table
+ *                    rows -- and a kernel expands it. Nothing is evaluated on
+ *                    the device, so nothing can round differently there.
  *
  * All tables are [seq, half] floats, half = sum of axis_dim / 2, one (cos, sin)
  * per rotated pair: the layout iris_dev_head_norm_rope takes. Column blocks
@@ -100,8 +102,8 @@ int iris_rope_qwen3_tables(float *cos_t, float *sin_t, const int *attention_mask
 
 /* ---- device-side generation (needs iris_dev_init) --------------------------------------- */
 
-/* Same arguments and meaning as the host builders above; d_cos / d_sin are device pointers from
- * iris_dev_alloc with room for rows * half floats. The work is enqueued on the backend's stream
+/* Same arguments, meaning and resulting bits as the host builders above; d_cos / d_sin are device
+ * pointers from iris_dev_alloc with room for rows * half floats. The work is enqueued on the backend's stream
  * like every other operator; pos / mask arguments are HOST arrays, read before the call returns.
  * Failures are reported as for the other iris_dev_* entries (one line on stderr,
  * iris_dev_last_error() non-zero). */

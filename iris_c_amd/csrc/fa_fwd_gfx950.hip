@@ -150,8 +150,8 @@ __device__ __forceinline__ int swz(int row) { return 2 * (row & 7); }
  * Written as asm, not as __builtin_amdgcn_global_load_lds: the compiler cannot tell which
  * stage a later LDS read touches and would wait for ALL outstanding requests (vmcnt(0))
  * before every operand read, which serialises the pipeline. The waits are placed by hand
- * (wait_vmcnt) where a tile is first needed. M0 carries the LDS address; nothing else in
- * this kernel uses M0. */
+ * (wait_vmcnt) where a tile is first needed. M0 carries the LDS address and is named as
+ * clobbered by every such statement. */
 __device__ __forceinline__ uint32_t lds_address(const uint16_t *p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
 }
@@ -163,6 +163,10 @@ __device__ __forceinline__ const uint16_t *scalar_ptr(const uint16_t *p) {
     return (const uint16_t *)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
 
+/* The compiler reserves M0 for its own short-lived uses and remarks on seeing it in a clobber list;
+ * naming it is still what tells it that a value it placed there does not survive the statement. */
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 template <int NI>
 __device__ __forceinline__ void load_tile(uint16_t *stage, const uint16_t *kt, const uint16_t *vt, int ldi,
                                           const uint32_t (&lane_off)[2], int wave) {
@@ -173,7 +177,7 @@ __device__ __forceinline__ void load_tile(uint16_t *stage, const uint16_t *kt, c
             const uint16_t *src = (g < 16 ? kt : vt) + (size_t)(4 * (g & 15)) * ldi;      /* first row of the piece */
             const uint16_t *dst = stage + (g < 16 ? 0 : K_TILE) + 4 * (g & 15) * KS;
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                         ::"s"(lds_address(dst)), "v"(lane_off[g & 1]), "s"(src) : "memory");
+                         ::"s"(lds_address(dst)), "v"(lane_off[g & 1]), "s"(src) : "memory", "m0");
         }
     } else {
         /* 16 or 32 pieces per wave (2 waves: one takes K, the other V; 1 wave: K then V). Source
@@ -189,7 +193,7 @@ __device__ __forceinline__ void load_tile(uint16_t *stage, const uint16_t *kt, c
 #pragma unroll
             for (int j = 0; j < 16; j++) {
                 asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                             ::"s"(dst), "v"(lane_off[j & 1]), "s"(src) : "memory");
+                             ::"s"(dst), "v"(lane_off[j & 1]), "s"(src) : "memory", "m0");
                 src += step;
                 dst += 4 * KS * 2;
                 asm volatile("" : "+s"(src), "+s"(dst));
@@ -213,9 +217,11 @@ __device__ __forceinline__ void load_tile_clamped(uint16_t *stage, const uint16_
         const uint16_t *src = (g < 16 ? kt : vt) + (size_t)min(row, last_row) * ldi + 8 * chunk;
         const uint16_t *dst = stage + (g < 16 ? 0 : K_TILE) + 4 * (g & 15) * KS;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                     ::"s"(lds_address(dst)), "v"(src) : "memory");
+                     ::"s"(lds_address(dst)), "v"(src) : "memory", "m0");
     }
 }
+
+#pragma clang diagnostic pop
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {

@@ -189,6 +189,10 @@ __device__ __forceinline__ uint32_t lds_address(const uint16_t *p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
 }
 
+/* M0 (the LDS address of a direct load) is named as clobbered by the asm statements below; the
+ * compiler reserves that register for its own short-lived uses and remarks on it. */
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 template <typename OUT, int TN, bool CONV>
 __global__ void __launch_bounds__(512, 2)
 k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *__restrict__ W,
@@ -243,7 +247,7 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
     }
     auto load16 = [&](uint16_t *dst, const uint16_t *src) {     /* per-lane source address */
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                     ::"s"(lds_address(dst)), "v"(src) : "memory");
+                     ::"s"(lds_address(dst)), "v"(src) : "memory", "m0");
     };
     auto request = [&](int kt, int stage) {
         uint16_t *w_dst = dlds + stage * STAGE + w_row0 * TK;
@@ -253,7 +257,7 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
 #pragma unroll
             for (int j = 0; j < W_PIECES; j++)
                 asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                             ::"s"(lds_address(w_dst + 8 * j * TK)), "v"(lane_off[j & 1]), "s"(src + (size_t)(8 * j) * K) : "memory");
+                             ::"s"(lds_address(w_dst + 8 * j * TK)), "v"(lane_off[j & 1]), "s"(src + (size_t)(8 * j) * K) : "memory", "m0");
         } else {
             /* rows past the end of the matrix are redirected to its last row (their outputs are never stored) */
 #pragma unroll
@@ -279,7 +283,7 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
 #pragma unroll
             for (int j = 0; j < X_PIECES; j++)
                 asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                             ::"s"(lds_address(x_dst + 8 * j * TK)), "v"(lane_off[j & 1]), "s"(src + (size_t)(8 * j) * K) : "memory");
+                             ::"s"(lds_address(x_dst + 8 * j * TK)), "v"(lane_off[j & 1]), "s"(src + (size_t)(8 * j) * K) : "memory", "m0");
         } else {
 #pragma unroll
             for (int j = 0; j < X_PIECES; j++) {
@@ -417,6 +421,7 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
         }
     }
 }
+#pragma clang diagnostic pop
 
 constexpr int DMA_LDS_BYTES = 128 * 1024;        /* two stages of (256 + 256) x 128 B; also the 8 x 16 KB of the epilogue */
 

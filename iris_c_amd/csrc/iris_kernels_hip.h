@@ -22,6 +22,10 @@ int iris_hip_norm_rope_hd128(void *stream, uint16_t *xq, uint16_t *xk, int ld,
                              const float *rope_cos, const float *rope_sin,
                              int seq, int q_heads, int k_heads, float eps, int split_half);
 
+/* The multiplier the kernel above divides by heads_total with (0 for one head, which needs
+ * none). Exported for the host-side test of the division. */
+uint32_t iris_norm_rope_magic(int heads_total);
+
 /* Any even head_dim <= 1024, any alignment. One wave per (token, head). */
 int iris_hip_norm_rope_generic(void *stream, uint16_t *x, int ld, const float *w,
                                const float *rope_cos, const float *rope_sin,
@@ -104,12 +108,12 @@ int iris_lt_linear(void *stream, void *y, int out_bf16, const uint16_t *x, const
 int iris_lt_available(void);
 void iris_lt_release(void);
 
-/* Rotary tables [seq, half] from positions [seq, naxes] (int32, or float when use_double) and
- * one frequency per column (float, or double when use_double); col_axis[half] names the axis of
- * each column. All pointers are device memory; freq 8-byte aligned when use_double. */
-int iris_hip_rope_tables(void *stream, float *cos_t, float *sin_t, const void *freq,
-                         const int *col_axis, const void *pos, int seq, int half, int naxes,
-                         int use_double);
+/* Rotary tables [seq, half] gathered from a dictionary of (axis, position) rows: entry
+ * (s, col) with columns[col] = (axis a, column j inside the axis, columns n of the axis, unused) is
+ * values[index[s * naxes + a] + j] for the cosine and ... + n + j for the sine. All pointers
+ * are device memory; columns is 16-byte aligned, index and values 4-byte aligned. */
+int iris_hip_rope_gather(void *stream, float *cos_t, float *sin_t, const float *values,
+                         const uint32_t *index, const void *columns, int seq, int half, int naxes);
 
 #ifdef __cplusplus
 }

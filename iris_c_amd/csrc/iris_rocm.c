@@ -36,7 +36,7 @@ static size_t g_gn_scratch_floats = 0;
 /* normalised copy of Q for the iris_dev_attention_qnorm calls that the matrix-core kernel does not take */
 static uint16_t *g_q_scratch = NULL;
 static size_t g_q_scratch_bytes = 0;
-/* positions and column frequencies of the rotary tables being generated */
+/* staging buffer of the rotary tables being expanded: column map, row offsets, dictionary */
 static void *g_rope_stage = NULL;
 static size_t g_rope_stage_bytes = 0;
 
@@ -430,8 +430,10 @@ void iris_dev_upsample2x(float *out, const float *in, int h, int width, int c) {
 
 /* ---- rotary tables generated on the device (include/iris_rope.h) ---- */
 
-/* Stages [freq: half x 8 B | col_axis: half x 4 B | pos: seq x naxes x 4 B] in one upload and
- * launches the table kernel. pos is int32 (use_double 0) or float (use_double 1). */
+/* The host evaluates every distinct (axis, position) of the sequence once, with the arithmetic
+ * of the host builders (iris_rope_tables.c), and stages [columns: half x 16 B | index: seq x
+ * naxes x 4 B | dictionary] in one upload; the kernel expands it into the two tables. pos is
+ * int32 (use_double 0) or float (use_double 1). */
 static void rope_tables(const char *what, float *d_cos, float *d_sin, const void *pos, int seq, int naxes,
                         const int *axis_dims, const int *axis_lens, float theta, int use_double) {
     if (!need_ready(what)) return;
@@ -442,24 +444,15 @@ static void rope_tables(const char *what, float *d_cos, float *d_sin, const void
     size_t half = 0;
     for (int a = 0; a < naxes; a++) half += (size_t)(axis_dims[a] / 2);
     if (!seq || !half) return;
-    const size_t freq_bytes = half * 8, axis_bytes = (half * 4 + 7) & ~(size_t)7;
-    const size_t pos_bytes = (size_t)seq * naxes * 4, total = freq_bytes + axis_bytes + pos_bytes;
-    unsigned char *blob = malloc(total);
-    if (!blob) { fail(-1, what, "out of host memory"); return; }
-    int *col_axis = (int *)(blob + freq_bytes);
-    size_t col = 0;
-    for (int a = 0; a < naxes; a++)
-        for (int j = 0; j < axis_dims[a] / 2; j++, col++) {
-            if (use_double) ((double *)blob)[col] = iris_rope_freq64_(theta, j, axis_dims[a]);
-            else ((float *)blob)[col] = iris_rope_freq32_(theta, j, axis_dims[a]);
-            col_axis[col] = a;
-        }
-    memcpy(blob + freq_bytes + axis_bytes, pos, pos_bytes);
-    if (axis_lens) {                       /* bounded axes: a position outside [0, len) does not rotate */
-        int *p = (int *)(blob + freq_bytes + axis_bytes);
-        for (size_t i = 0; i < (size_t)seq * naxes; i++)
-            if (p[i] < 0 || p[i] >= axis_lens[i % naxes]) p[i] = 0;
+    float *values = NULL;
+    uint32_t *index = NULL;
+    size_t n_values = 0;
+    if (iris_rope_dictionary_(pos, use_double, seq, naxes, axis_dims, axis_lens, theta, &values, &n_values, &index) != 0) {
+        fail(-1, what, "out of host memory");
+        return;
     }
+    const size_t col_bytes = half * 16, idx_bytes = (size_t)seq * naxes * 4, val_bytes = n_values * 4;
+    const size_t total = col_bytes + idx_bytes + val_bytes;
     if (total > g_rope_stage_bytes) {
         if (g_rope_stage) {
             check(hipStreamSynchronize(g_stream), "sync");
@@ -470,20 +463,30 @@ static void rope_tables(const char *what, float *d_cos, float *d_sin, const void
         if (hipMalloc(&g_rope_stage, total) != hipSuccess) {
             (void)hipGetLastError();
             g_rope_stage = NULL;
-            free(blob);
-            fail(-1, what, "out of device memory for the position staging buffer");
+            free(values); free(index);
+            fail(-1, what, "out of device memory for the staging buffer");
             return;
         }
         g_rope_stage_bytes = total;
     }
+    unsigned char *blob = malloc(total);
+    if (!blob) { free(values); free(index); fail(-1, what, "out of host memory"); return; }
+    int *col = (int *)blob;
+    for (int a = 0; a < naxes; a++)
+        for (int j = 0; j < axis_dims[a] / 2; j++, col += 4) {
+            col[0] = a; col[1] = j; col[2] = axis_dims[a] / 2; col[3] = 0;
+        }
+    memcpy(blob + col_bytes, index, idx_bytes);
+    memcpy(blob + col_bytes + idx_bytes, values, val_bytes);
+    free(values); free(index);
     /* stream order keeps an earlier table kernel's reads ahead of this overwrite of the staging buffer */
     int ok = check(hipMemcpyAsync(g_rope_stage, blob, total, hipMemcpyHostToDevice, g_stream), "upload") &&
              check(hipStreamSynchronize(g_stream), "sync");
     free(blob);
     if (!ok) return;
     const unsigned char *d = g_rope_stage;
-    int err = iris_hip_rope_tables(g_stream, d_cos, d_sin, d, (const int *)(d + freq_bytes),
-                                   d + freq_bytes + axis_bytes, seq, (int)half, naxes, use_double);
+    int err = iris_hip_rope_gather(g_stream, d_cos, d_sin, (const float *)(d + col_bytes + idx_bytes),
+                                   (const uint32_t *)(d + col_bytes), d, seq, (int)half, naxes);
     if (err) check((hipError_t)err, "rope tables launch");
 }
 

@@ -6,8 +6,13 @@
 #ifndef IRIS_ROPE_INTERNAL_H
 #define IRIS_ROPE_INTERNAL_H
 
-float iris_rope_freq32_(float theta, int j, int dim);
-double iris_rope_freq64_(float theta, int j, int dim);
+#include <stddef.h>
+#include <stdint.h>
+
+/* A table as a dictionary of its distinct (axis, position) rows plus one offset per (row, axis);
+ * see iris_rope_tables.c. values and index are malloc'd. */
+int iris_rope_dictionary_(const void *pos, int use_double, int seq, int naxes, const int *axis_dims,
+                          const int *axis_lens, float theta, float **values, size_t *n_values, uint32_t **index);
 /* malloc'd positions of the text encoder's rows, NULL on failure */
 int *iris_rope_qwen3_positions_(const int *attention_mask, int seq, int pad_at_one);
 /* argument check of the expansion routines: 1 = usable */

@@ -45,8 +45,8 @@ typedef struct {
 } axis_memo;
 
 /* the one place the column frequencies are written down */
-float iris_rope_freq32_(float theta, int j, int dim) { return 1.0f / powf(theta, (float)(2 * j) / (float)dim); }
-double iris_rope_freq64_(float theta, int j, int dim) { return 1.0 / pow(theta, (double)(2 * j) / dim); }
+static float iris_rope_freq32_(float theta, int j, int dim) { return 1.0f / powf(theta, (float)(2 * j) / (float)dim); }
+static double iris_rope_freq64_(float theta, int j, int dim) { return 1.0 / pow(theta, (double)(2 * j) / dim); }
 
 static void memo_free(axis_memo *m, int naxes) {
     for (int a = 0; a < naxes; a++) {
@@ -76,22 +76,27 @@ static int memo_init(axis_memo *m, int naxes, const int *axis_dims, float theta,
     return 1;
 }
 
+/* The one place a table entry is evaluated: cos row then sin row of one (axis, position). */
+static void eval_row(float *row, int cols, const float *freq32, const double *freq64, float value, int use_double) {
+    for (int j = 0; j < cols; j++) {
+        if (use_double) {
+            const double angle = value * freq64[j];
+            row[j] = (float)cos(angle);
+            row[cols + j] = (float)sin(angle);
+        } else {
+            const float angle = value * freq32[j];
+            row[j] = cosf(angle);
+            row[cols + j] = sinf(angle);
+        }
+    }
+}
+
 /* cos / sin rows of one (axis, position); bits identify the position, value is what is multiplied */
 static const float *memo_row(axis_memo *m, uint32_t bits, float value, int use_double) {
     const uint32_t slot = (bits * 2654435761u) >> 22;          /* top 10 bits of a Fibonacci hash */
     float *row = m->cs + (size_t)slot * 2 * m->cols;
     if (m->used[slot] && m->key[slot] == bits) return row;
-    for (int j = 0; j < m->cols; j++) {
-        if (use_double) {
-            const double angle = value * m->freq64[j];
-            row[j] = (float)cos(angle);
-            row[m->cols + j] = (float)sin(angle);
-        } else {
-            const float angle = value * m->freq32[j];
-            row[j] = cosf(angle);
-            row[m->cols + j] = sinf(angle);
-        }
-    }
+    eval_row(row, m->cols, m->freq32, m->freq64, value, use_double);
     m->used[slot] = 1;
     m->key[slot] = bits;
     return row;
@@ -148,6 +153,71 @@ int iris_rope_expand_f64(float *cos_t, float *sin_t, const float *pos, int seq, 
         }
     }
     memo_free(memo, naxes);
+    return 0;
+}
+
+/* ---- dictionary form, for the device entries ------------------------------------------------ */
+
+/* The same table as a dictionary: `values` holds, for every distinct (axis, position) of the
+ * sequence, the cos row and the sin row of that axis (2 * axis_dim / 2 floats, evaluated by
+ * eval_row like the tables above), and index[s * naxes + a] is the offset in floats of the pair of
+ * rows that row s uses on axis a. Expanding it is pure copying, so a table gathered from the
+ * dictionary has the bits of the table built here directly. pos is int32 [seq][naxes]
+ * (use_double 0, axis_lens as in iris_rope_expand_i32) or float (use_double 1). Returns 0 and
+ * malloc'd arrays, or -1. */
+int iris_rope_dictionary_(const void *pos, int use_double, int seq, int naxes, const int *axis_dims,
+                          const int *axis_lens, float theta, float **values, size_t *n_values, uint32_t **index) {
+    axis_memo memo[MAX_AXES];
+    *values = NULL; *index = NULL; *n_values = 0;
+    if (!axes_ok(seq, naxes, axis_dims) || (seq && !pos)) return -1;
+    if (!memo_init(memo, naxes, axis_dims, theta, use_double)) return -1;
+    /* open-addressing map position bits -> offset, one per axis, at most half full */
+    size_t cap = 16;
+    while (cap < 2 * (size_t)seq) cap <<= 1;
+    uint32_t *keys = malloc(sizeof(uint32_t) * cap), *offs = malloc(sizeof(uint32_t) * cap);
+    unsigned char *used = malloc(cap);
+    uint32_t *idx = malloc(sizeof(uint32_t) * (size_t)(seq ? seq : 1) * (size_t)naxes);
+    size_t room = 1024, n = 0;
+    float *vals = malloc(sizeof(float) * room);
+    int ok = keys && offs && used && idx && vals;
+    for (int a = 0; ok && a < naxes; a++) {
+        const int cols = memo[a].cols;
+        memset(used, 0, cap);
+        for (int s = 0; ok && s < seq; s++) {
+            uint32_t bits;
+            float value;
+            if (use_double) {
+                value = ((const float *)pos)[(size_t)s * naxes + a];
+                memcpy(&bits, &value, sizeof bits);
+            } else {
+                int p = ((const int *)pos)[(size_t)s * naxes + a];
+                if (axis_lens && (p < 0 || p >= axis_lens[a])) p = 0;     /* out of range: unrotated */
+                bits = (uint32_t)p;
+                value = (float)p;
+            }
+            size_t slot = (size_t)((bits * 2654435761u) >> 4) & (cap - 1);
+            while (used[slot] && keys[slot] != bits) slot = (slot + 1) & (cap - 1);
+            if (!used[slot]) {
+                if (n + 2 * (size_t)cols > room) {
+                    while (n + 2 * (size_t)cols > room) room *= 2;
+                    float *grown = realloc(vals, sizeof(float) * room);
+                    if (!grown) { ok = 0; break; }
+                    vals = grown;
+                }
+                if (n + 2 * (size_t)cols >= 0x80000000u) { ok = 0; break; }    /* offsets are 32 bits */
+                eval_row(vals + n, cols, memo[a].freq32, memo[a].freq64, value, use_double);
+                used[slot] = 1;
+                keys[slot] = bits;
+                offs[slot] = (uint32_t)n;
+                n += 2 * (size_t)cols;
+            }
+            idx[(size_t)s * naxes + a] = offs[slot];
+        }
+    }
+    memo_free(memo, naxes);
+    free(keys); free(offs); free(used);
+    if (!ok) { free(idx); free(vals); return -1; }
+    *values = vals; *n_values = n; *index = idx;
     return 0;
 }
 

@@ -88,7 +88,8 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
         int unit = first + u * (kThreads / 16);
         const bool live = unit < units;
         unit = live ? unit : 0;
-        const int s = (int)__umulhi((uint32_t)unit, magic);       /* unit / heads_total */
+        /* unit / heads_total; one head per token has no 32-bit magic (it would be 2^32) */
+        const int s = heads_total == 1 ? unit : (int)__umulhi((uint32_t)unit, magic);
         const int h = unit - s * heads_total;
         isk[u] = h >= q_heads;
         uint16_t *base = isk[u] ? xk + (size_t)(h - q_heads) * 128 : xq + (size_t)h * 128;
@@ -183,6 +184,14 @@ k_norm_rope_generic(uint16_t *x, int ld, const float *w, const float *rope_cos,
 
 }  // namespace
 
+/* unit / heads_total == umulhi(unit, magic) for unit < 2^24 and 2 <= heads_total < 2^8. For one
+ * head the constant would be 2^32, which does not fit: 0 is returned and the kernel takes
+ * unit / 1 = unit without it. */
+extern "C" uint32_t iris_norm_rope_magic(int heads_total) {
+    if (heads_total <= 1) return 0u;
+    return (uint32_t)((0x100000000ull + (uint64_t)heads_total - 1) / (uint64_t)heads_total);
+}
+
 extern "C" int iris_hip_norm_rope_hd128(void *stream, uint16_t *xq, uint16_t *xk, int ld,
                                         const float *wq, const float *wk,
                                         const float *rope_cos, const float *rope_sin,
@@ -191,8 +200,7 @@ extern "C" int iris_hip_norm_rope_hd128(void *stream, uint16_t *xq, uint16_t *xk
     const int heads_total = q_heads + k_heads;
     const int units = seq * heads_total;
     if (units <= 0) return 0;
-    /* unit / heads_total == umulhi(unit, magic) for unit < 2^24, heads_total < 2^8 */
-    const uint32_t magic = (uint32_t)((0x100000000ull + heads_total - 1) / heads_total);
+    const uint32_t magic = iris_norm_rope_magic(heads_total);
     const int blocks = (units + kUnitsPerBlock - 1) / kUnitsPerBlock;
     hipStream_t st = (hipStream_t)stream;
     if (split_half)

@@ -1,8 +1,8 @@
 """numpy mirror of include/iris_rope.h: the rotary-table builders of libiris_dev.so.
 
 Host builders need no GPU (the functions are plain C + libm inside the same
-library); the `dev_*` forms take an `IrisDev` and return the table generated
-on the device, downloaded. Used by tests and the benchmark only.
+library); the `dev_*` forms take an `IrisDev` and return the table expanded on
+the device, downloaded. Used by tests and the benchmark only.
 """
 import ctypes as C
 
@@ -104,6 +104,38 @@ class RopeTables:
         rc = self.lib.iris_rope_qwen3_tables(_p(c), _p(s), _p(_ints(mask)), seq, head_dim, theta, int(pad_at_one))
         assert rc == 0
         return c, s
+
+
+    # ---- the dictionary the device entries upload (internal symbol; for the tests of that path)
+    def dictionary(self, pos, axis_dims, theta, axis_lens=None, use_double=False):
+        """(values, index): distinct (axis, position) rows and one offset per (row, axis)."""
+        dims, lens = _ints(axis_dims), _ints(axis_lens)
+        pos = (np.ascontiguousarray(pos, np.float32) if use_double else _ints(pos)).reshape(-1, len(dims))
+        fn = self.lib.iris_rope_dictionary_
+        fn.restype = C.c_int
+        fn.argtypes = [_vp, C.c_int, C.c_int, C.c_int, _vp, _vp, C.c_float, C.POINTER(_vp), C.POINTER(C.c_size_t),
+                       C.POINTER(_vp)]
+        values, index, n = _vp(), _vp(), C.c_size_t()
+        rc = fn(_p(pos), int(use_double), len(pos), len(dims), _p(dims), _p(lens), theta, C.byref(values), C.byref(n),
+                C.byref(index))
+        if rc != 0:
+            return rc, None, None
+        libc = C.CDLL(None)
+        libc.free.argtypes = [_vp]
+        v = np.ctypeslib.as_array(C.cast(values, C.POINTER(C.c_float)), shape=(max(n.value, 1),))[:n.value].copy()
+        i = np.ctypeslib.as_array(C.cast(index, C.POINTER(C.c_uint32)), shape=(max(pos.size, 1),))[:pos.size].copy()
+        libc.free(values); libc.free(index)
+        return 0, v, i.reshape(pos.shape)
+
+    @staticmethod
+    def expand_dictionary(values, index, axis_dims):
+        """What the device kernel does, in numpy."""
+        cos_t, sin_t = [], []
+        for a, d in enumerate(axis_dims):
+            n = d // 2
+            at = index[:, a].astype(np.int64)[:, None] + np.arange(n)[None, :]
+            cos_t.append(values[at]); sin_t.append(values[at + n])
+        return np.concatenate(cos_t, axis=1), np.concatenate(sin_t, axis=1)
 
 
 class DevRopeTables(RopeTables):

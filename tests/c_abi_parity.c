@@ -27,16 +27,24 @@
 
 static int failures = 0;
 
+/* Absolute bar (max_tol, mean_tol) and, so that small outputs are held as tightly as large ones,
+ * the same errors against the size of the expected values: max-abs <= 4e-2 max|want|,
+ * mean-abs <= 1e-2 mean|want|. An all-zero reference is refused. */
 static void compare(const char *what, const uint16_t *got, const float *want, size_t n,
                     double max_tol, double mean_tol) {
-    double mx = 0.0, sum = 0.0;
+    double mx = 0.0, sum = 0.0, ref_mx = 0.0, ref_sum = 0.0;
     for (size_t i = 0; i < n; i++) {
         double d = fabs((double)orc_bf2f(got[i]) - (double)want[i]);
         if (!(d <= mx)) mx = d;                    /* also catches NaN */
         sum += d;
+        double w = fabs((double)want[i]);
+        if (w > ref_mx) ref_mx = w;
+        ref_sum += w;
     }
-    int ok = mx <= max_tol && sum / (double)n <= mean_tol;
-    printf("%-34s max-abs %.3e  mean-abs %.3e  %s\n", what, mx, sum / (double)n, ok ? "ok" : "FAIL");
+    const double mean = sum / (double)n, ref_mean = ref_sum / (double)n;
+    int ok = mx <= max_tol && mean <= mean_tol && ref_mean > 0.0 && mx <= 4e-2 * ref_mx && mean <= 1e-2 * ref_mean;
+    printf("%-34s max-abs %.3e (max|want| %.3e)  mean-abs %.3e (mean|want| %.3e)  %s\n", what, mx, ref_mx, mean,
+           ref_mean, ok ? "ok" : "FAIL");
     if (!ok) failures++;
 }
 

@@ -95,3 +95,27 @@ def test_unmodified_reference_links_against_this_backend(lib):
     assert set(used) <= set(iris_c_amd.ABI), sorted(set(used) - set(iris_c_amd.ABI))
     ldd = subprocess.run(["ldd", exe], capture_output=True, text=True, check=True).stdout
     assert "libiris_dev.so" in ldd and "not found" not in ldd
+
+
+def test_division_constant_of_the_norm_rope_kernel(lib):
+    """The fast norm+rope kernel turns a unit index into (token, head) with one multiply-high by
+    the constant its launcher computes (0 = "one head, no division"). Checked the way the kernel
+    uses it, over the whole range the dispatcher admits: unit < 2^24, 1 <= heads < 256."""
+    import ctypes as C
+    import numpy as np
+    magic = lib.iris_norm_rope_magic
+    magic.restype, magic.argtypes = C.c_uint32, [C.c_int]
+    assert magic(1) == 0                               # 2^32 does not fit: the kernel takes unit / 1 = unit
+    top = 1 << 24
+    edge = np.array([0, 1, 2, top - 2, top - 1], dtype=np.uint64)
+    for d in range(2, 256):
+        m = np.uint64(magic(d))
+        assert 0 < m < (1 << 32)
+        if d in (2, 3, 24, 30, 32, 40, 48, 60, 64, 96, 255):
+            units = np.arange(top, dtype=np.uint64)    # every admitted unit
+        else:                                          # multiples of d and their neighbours, a stride, the ends
+            mult = np.arange(0, top, d, dtype=np.uint64)[-4096:]
+            units = np.unique(np.concatenate([edge, mult, mult - np.uint64(1), mult[:-1] + np.uint64(d - 1),
+                                              np.arange(0, top, 4099, dtype=np.uint64), np.arange(70000, dtype=np.uint64)]))
+            units = units[units < top]
+        assert np.array_equal((units * m) >> np.uint64(32), units // np.uint64(d)), d

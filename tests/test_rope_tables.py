@@ -142,6 +142,50 @@ def test_reuse_of_positions_never_changes_a_value(rt):
         assert same_bits(c[i], c1[0]) and same_bits(s[i], s1[0])
 
 
+def test_dictionary_form_expands_to_the_same_bits(rt, gold):
+    """The device entries upload a dictionary of the distinct (axis, position) rows plus one offset per
+    (token, axis), and a kernel expands it. Expanded here in numpy: it must give the bits of the direct
+    builders, hold each distinct position once, and match the reference's golden tables."""
+    # FLUX.2 joint layout: text + image + two reference images
+    pos = rt.flux2_positions(8, 4, 5, REFS)
+    rc, values, index = rt.dictionary(pos, (32, 32, 32, 32), 2000.0)
+    assert rc == 0
+    c, s = rt.expand_dictionary(values, index, (32, 32, 32, 32))
+    assert same_bits(c, gold["flux2_cos"]) and same_bits(s, gold["flux2_sin"])
+    distinct = sum(len(np.unique(pos[:, a])) for a in range(4))
+    assert values.size == distinct * 32                      # 16 cos + 16 sin per distinct (axis, position)
+    # FLUX.3: float positions, double arithmetic
+    fpos = rt.flux3_positions(8, 4, 5, REFS)
+    rc, values, index = rt.dictionary(fpos, (32, 32, 32, 32), 10000.0, use_double=True)
+    c, s = rt.expand_dictionary(values, index, (32, 32, 32, 32))
+    assert rc == 0 and same_bits(c, gold["flux3_cos"]) and same_bits(s, gold["flux3_sin"])
+    # Z-Image: bounded axes, uneven axis sizes; many rows, few positions
+    zpos, _, _, _ = rt.zimage_positions(img_seq=1000, wt=40, cap_seq=77)
+    lens = (64, 20, 512)
+    rc, values, index = rt.dictionary(zpos, (32, 48, 48), 256.0, axis_lens=lens)
+    c, s = rt.expand_dictionary(values, index, (32, 48, 48))
+    hc, hs = rt.zimage_tables(zpos, (32, 48, 48), lens)
+    assert rc == 0 and same_bits(c, hc) and same_bits(s, hs)
+    assert values.size * 4 < c.nbytes // 10                 # the point of the form: far smaller than the tables
+    # every position distinct (text encoder): the dictionary is the table
+    rc, values, index = rt.dictionary(np.arange(3000, dtype=np.int32), (128,), 1e6)
+    c, s = rt.expand_dictionary(values, index, (128,))
+    hc, hs = rt.qwen3_tables(3000, 128, 1e6)
+    assert rc == 0 and same_bits(c, hc) and same_bits(s, hs) and values.size == 3000 * 128
+    # random positions incl. collisions in the position map
+    g = np.random.default_rng(8)
+    rpos = g.integers(0, 50000, size=(5000, 3)).astype(np.int32)
+    rpos[::5] = rpos[3]
+    rc, values, index = rt.dictionary(rpos, (16, 40, 72), 500.0)
+    c, s = rt.expand_dictionary(values, index, (16, 40, 72))
+    rc2, hc, hs = rt.expand_i32(rpos, (16, 40, 72), 500.0)
+    assert rc == 0 and rc2 == 0 and same_bits(c, hc) and same_bits(s, hs)
+    # refused arguments
+    assert rt.dictionary(rpos, (15, 40, 72), 500.0)[0] == -1
+    rc, values, index = rt.dictionary(np.zeros((0, 2), np.int32), (32, 32), 100.0)
+    assert rc == 0 and values.size == 0
+
+
 def test_closed_form(rt):
     """cos / sin of p * theta^(-2j/d), evaluated in double, within float rounding of the angle."""
     pos = np.array([[0, 1], [3, 250], [4095, 17]], np.int32)
