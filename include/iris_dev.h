@@ -118,6 +118,15 @@ void iris_dev_conv2d(float *out, const float *in, const uint16_t *w, const float
  * (reference iris_dev.h:123-126) */
 void iris_dev_group_norm(float *out, const float *in, const float *gamma, const float *beta,
                          int hw, int c, int groups, float eps, int silu);
+/* No counterpart in the reference. The same operator for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * same arguments, same kernels and the same bits as iris_dev_group_norm, but its scratch (partial
+ * moments and statistics, 787 KB) is an array inside the library instead of memory allocated at
+ * the first call, so this entry calls no hipMalloc / hipFree at all. groups <= 64; more is refused
+ * with an error (use iris_dev_group_norm). All calls on a GPU share that one array: calls that
+ * overlap in time would race, so keep them on the library's stream, which orders them. */
+void iris_dev_group_norm_noalloc(float *out, const float *in, const float *gamma, const float *beta,
+                                 int hw, int c, int groups, float eps, int silu);
 /* nearest-neighbour 2x upsampling of [h * w, c] into [2h * 2w, c] (reference iris_dev.h:128-129) */
 void iris_dev_upsample2x(float *out, const float *in, int h, int width, int c);
 

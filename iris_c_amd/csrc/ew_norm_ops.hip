@@ -9,8 +9,11 @@
  * no barrier) and keep the row in registers between the statistics and the
  * write (rows up to 4096 floats; longer rows are read again, from cache).
  * Statistics follow the reference: LayerNorm takes the mean first and the
- * variance about it. Group norm does the same in two passes over the image
- * with coalesced per-pixel reads and per-group partial sums.
+ * variance about it. Group norm takes its statistics in ONE pass over the
+ * image (coalesced per-pixel reads, per-workgroup partial moments of every
+ * group, merged in double by a small second kernel) and normalises in a
+ * second pass; the partial moments and the final statistics live in a
+ * scratch buffer the caller of the launcher provides.
  */
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -491,7 +494,8 @@ int iris_hip_rms_norm_residual(void *stream, float *x, const float *a, const flo
 
 size_t iris_hip_group_norm_scratch_floats(int groups) { return 3 * (size_t)groups * GN_MAX_BLOCKS + 2 * (size_t)groups; }
 
-/* scratch: iris_hip_group_norm_scratch_floats(groups) floats of device memory */
+/* scratch: iris_hip_group_norm_scratch_floats(groups) floats of device memory. Every slot a call
+ * reads (partial moments [group][workgroup], statistics [2][group]) is written by that call first. */
 int iris_hip_group_norm(void *stream, float *scratch, float *out, const float *in, const float *gamma,
                         const float *beta, int hw, int c, int groups, float eps, int do_silu) {
     if (hw <= 0 || c <= 0) return 0;
@@ -521,6 +525,55 @@ int iris_hip_group_norm(void *stream, float *scratch, float *out, const float *i
     else
         hipLaunchKernelGGL(k_gn_normalize<1>, dim3(blocks_for(n, EW_THREADS)), dim3(EW_THREADS), 0, st, out, in, stats, gamma, beta, c, cg, groups, do_silu, n);
     return (int)hipGetLastError();
+}
+
+}  // extern "C"
+
+/* ---- group norm for callers that cannot allocate -------------------------------------------
+ * The same kernels with their scratch in a device array that is part of the library image, so the
+ * call needs no hipMalloc: each GPU holds its own copy of the array, at its own address, until the
+ * process ends. In host code the array's name is only a handle for hipGetSymbolAddress; kernels
+ * get the address that call returned, kept per device. Calls on one GPU share the array: they must
+ * not overlap (the library issues everything on one stream, which orders them). */
+constexpr int GN_STATIC_MAX_GROUPS = 64;
+constexpr size_t GN_STATIC_FLOATS = 3 * (size_t)GN_STATIC_MAX_GROUPS * GN_MAX_BLOCKS + 2 * (size_t)GN_STATIC_MAX_GROUPS;
+static __device__ __align__(256) float scratch[GN_STATIC_FLOATS];          /* 786,944 B */
+
+constexpr int GN_STATIC_MAX_DEVICES = 64;
+static float *scratch_address[GN_STATIC_MAX_DEVICES];                        /* per device; null = not looked up yet */
+
+extern "C" {
+
+int iris_hip_group_norm_static_max_groups(void) { return GN_STATIC_MAX_GROUPS; }
+
+/* Looks up the address of the current device's copy of the array (once per device). */
+int iris_hip_group_norm_static_setup(void) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= GN_STATIC_MAX_DEVICES) return (int)hipErrorInvalidDevice;
+    if (scratch_address[dev]) return 0;
+    float *p = nullptr;
+    e = hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return (int)hipErrorInvalidSymbol;
+    scratch_address[dev] = p;
+    return 0;
+}
+
+/* groups <= iris_hip_group_norm_static_max_groups(), checked by the caller too */
+int iris_hip_group_norm_static(void *stream, float *out, const float *in, const float *gamma,
+                               const float *beta, int hw, int c, int groups, float eps, int do_silu) {
+    if (groups <= 0 || groups > GN_STATIC_MAX_GROUPS) return (int)hipErrorInvalidValue;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= GN_STATIC_MAX_DEVICES) return (int)hipErrorInvalidDevice;
+    if (!scratch_address[dev]) {                         /* first call on a device the set-up call did not see */
+        const int rc = iris_hip_group_norm_static_setup();
+        if (rc) return rc;
+    }
+    return iris_hip_group_norm(stream, scratch_address[dev], out, in, gamma, beta, hw, c, groups, eps, do_silu);
 }
 
 }  // extern "C"

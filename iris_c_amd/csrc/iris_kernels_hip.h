@@ -86,6 +86,14 @@ size_t iris_hip_group_norm_scratch_floats(int groups);
 int iris_hip_group_norm(void *stream, float *scratch, float *out, const float *in, const float *gamma,
                         const float *beta, int hw, int c, int groups, float eps, int do_silu);
 
+/* The same with the scratch in a device array inside the library (no allocation anywhere):
+ * groups <= iris_hip_group_norm_static_max_groups(). The set-up call looks up the array's address
+ * on the current device, once per device; the launcher does it itself on a device it has not seen. */
+int iris_hip_group_norm_static_max_groups(void);
+int iris_hip_group_norm_static_setup(void);
+int iris_hip_group_norm_static(void *stream, float *out, const float *in, const float *gamma,
+                               const float *beta, int hw, int c, int groups, float eps, int do_silu);
+
 /* ---- linear layers and convolution (gemm_conv_gfx950.hip) ---- */
 /* y[rows, out] = x[rows, in] @ W[out, in]^T, contiguous; MFMA kernel when in % 8 == 0 and
  * x, W are 16-byte aligned, scalar kernel otherwise */

@@ -73,6 +73,9 @@ int iris_dev_init(void) {
     snprintf(g_name, sizeof(g_name), "%s (%s, %d CUs, %d MHz)", prop.name[0] ? prop.name : "AMD Instinct",
              prop.gcnArchName, prop.multiProcessorCount, prop.clockRate / 1000);
     if (hipStreamCreate(&g_stream) != hipSuccess) return 0;
+    /* address of the in-library scratch of iris_dev_group_norm_noalloc on this device; if the lookup
+     * fails here the entry point tries again at its first call and reports it there */
+    (void)iris_hip_group_norm_static_setup();
     g_ready = 1;
     g_last_error = 0;
     return 1;
@@ -421,6 +424,20 @@ void iris_dev_group_norm(float *out, const float *in, const float *gamma, const 
     }
     int err = iris_hip_group_norm(g_stream, g_gn_scratch, out, in, gamma, beta, hw, c, groups, eps, silu != 0);
     if (err) check((hipError_t)err, "group_norm launch");
+}
+
+/* The same operator for callers that cannot allocate: scratch is an array inside the library. */
+void iris_dev_group_norm_noalloc(float *out, const float *in, const float *gamma, const float *beta,
+                                 int hw, int c, int groups, float eps, int silu) {
+    if (!need_ready("group_norm_noalloc")) return;
+    if (hw <= 0 || c <= 0) return;
+    if (groups <= 0 || c % groups != 0) { fail(-1, "group_norm_noalloc", "need c % groups == 0"); return; }
+    if (groups > iris_hip_group_norm_static_max_groups()) {
+        fail(-1, "group_norm_noalloc", "more than 64 groups: beyond the built-in scratch, use iris_dev_group_norm");
+        return;
+    }
+    int err = iris_hip_group_norm_static(g_stream, out, in, gamma, beta, hw, c, groups, eps, silu != 0);
+    if (err) check((hipError_t)err, "group_norm_noalloc launch");
 }
 
 void iris_dev_upsample2x(float *out, const float *in, int h, int width, int c) {

@@ -63,6 +63,8 @@ def test_no_gpu_means_no_silent_fallback(lib):
     assert lib.iris_dev_last_error() != 0
     lib.iris_dev_conv2d(None, None, None, None, 4, 4, 64, 128, 3, 1, 1, 1)
     assert lib.iris_dev_last_error() != 0
+    lib.iris_dev_group_norm_noalloc(None, None, None, None, 4, 8, 2, 1e-6, 0)
+    assert lib.iris_dev_last_error() != 0
     # device-side table generation likewise; the host builders of the same header need no device
     lib.iris_dev_rope_qwen3_tables(None, None, None, 4, 128, 1e6, 0)
     assert lib.iris_dev_last_error() != 0
