@@ -96,7 +96,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
-/* A workgroup is WAVES (4 or 8) waves of 32 queries: BM = 32 * WAVES queries, 64 * WAVES threads. */
+/* A workgroup is WAVES waves of NB blocks of 16 queries (NB = 2 in every launch): BM = 16 * NB * WAVES queries,
+ * 64 * WAVES threads. */
 constexpr int BN = 64;             /* keys per tile */
 constexpr int HD = 128;
 constexpr int KS = HD;              /* K and V tile rows are 256 B, unpadded: chunks are swizzled instead */
@@ -121,10 +122,11 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2));
 }
 
+/* v_maximum3_f32 (a -inf operand is an ordinary value to it). As a builtin, not as inline asm: the
+ * compiler may then interleave the independent chains of the two query blocks and place the
+ * hazard gaps itself. */
 __device__ __forceinline__ float max3(float a, float b, float c) {
-    float d;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
-    return d;
+    return __builtin_elementwise_maximum(__builtin_elementwise_maximum(a, b), c);
 }
 
 /* Max over the four lanes l%16, l%16+16, +32, +48 (one per 16-lane row); every one
@@ -141,7 +143,7 @@ __device__ __forceinline__ int swz(int row) { return 2 * (row & 7); }
 
 /* HBM/L2 -> LDS without passing through registers: one global_load_lds_dwordx4 moves
  * 64 lanes x 16 B into 1 KB of consecutive LDS (lane l at +16 l), i.e. four tile rows.
- * A tile (K then V, 32 KB) is 32 such pieces, NI = 32 / WAVES per wave; piece g covers
+ * A tile (K then V, 32 KB) is 32 such pieces, NI = ceil(32 / WAVES) per wave; piece g covers
  * rows 4 (g % 16) .. +3 of K (g < 16) or V. The lane that fills slot s of row r fetches
  * chunk s ^ swz(r) of that row: the swizzle is applied on the source side. Rows r and
  * r + 8 swizzle alike, so a lane needs two source offsets in all: lane_off[g % 2], from
@@ -167,13 +169,16 @@ __device__ __forceinline__ const uint16_t *scalar_ptr(const uint16_t *p) {
  * naming it is still what tells it that a value it placed there does not survive the statement. */
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-template <int NI>
+template <int NI, int WAVES>
 __device__ __forceinline__ void load_tile(uint16_t *stage, const uint16_t *kt, const uint16_t *vt, int ldi,
                                           const uint32_t (&lane_off)[2], int wave) {
     if constexpr (NI <= 8) {
 #pragma unroll
         for (int j = 0; j < NI; j++) {
-            const int g = wave * NI + j;                       /* wave-uniform */
+            /* wave-uniform. A wave count that does not divide 32 (12 waves) deals the pieces out
+             * round-robin, and the last round is short. */
+            const int g = 32 % WAVES == 0 ? wave * NI + j : wave + j * WAVES;
+            if (32 % WAVES != 0 && g >= 32) break;
             const uint16_t *src = (g < 16 ? kt : vt) + (size_t)(4 * (g & 15)) * ldi;      /* first row of the piece */
             const uint16_t *dst = stage + (g < 16 ? 0 : K_TILE) + 4 * (g & 15) * KS;
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -206,12 +211,13 @@ __device__ __forceinline__ void load_tile(uint16_t *stage, const uint16_t *kt, c
  * past `last_row` (relative to the tile) are redirected to it. Their scores are masked and
  * their probabilities are exactly zero, so the values never matter; they only must be
  * finite, which any real row is. */
-template <int NI>
+template <int NI, int WAVES>
 __device__ __forceinline__ void load_tile_clamped(uint16_t *stage, const uint16_t *kt, const uint16_t *vt, int ldi,
                                                   int last_row, int lane, int wave) {
 #pragma unroll
     for (int j = 0; j < NI; j++) {
-        const int g = wave * NI + j;
+        const int g = 32 % WAVES == 0 ? wave * NI + j : wave + j * WAVES;
+        if (32 % WAVES != 0 && g >= 32) break;
         const int row = 4 * (g & 15) + (lane >> 4);
         const int chunk = (lane & 15) ^ swz(row);
         const uint16_t *src = (g < 16 ? kt : vt) + (size_t)min(row, last_row) * ldi + 8 * chunk;
@@ -309,18 +315,20 @@ __device__ __forceinline__ void norm_rope_q_fragment(bf16x8 (&qb)[4], const QNor
                                                   pack_bf16(o[ks][4], o[ks][5]), pack_bf16(o[ks][6], o[ks][7])});
 }
 
-template <int WAVES, bool CAUSAL, bool MASK>
+
+template <int WAVES, int NB, bool CAUSAL, bool MASK>
 __global__ void __launch_bounds__(64 * WAVES, 2)
 k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ q,
                const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
                int seq_q, int seq_k, int q_tiles, int total_work, int work_per_xcd,
                int kv_group, float scale_log2, const int *__restrict__ key_mask, QNorm qnorm) {
     extern __shared__ __align__(16) uint16_t lds[];     /* NSTAGE stages of [K tile | V tile] */
-    constexpr int BM = 32 * WAVES, NI = 32 / WAVES;
+    constexpr int WQ = 16 * NB;                          /* queries per wave: NB blocks of 16 */
+    constexpr int BM = WQ * WAVES, NI = (32 + WAVES - 1) / WAVES;   /* pieces of a tile per wave (the last waves may have one fewer) */
     /* Key tiles between two barriers. Two for the 8-wave shape (one workgroup per CU, so the LDS
      * has room for four stages): the waves of a workgroup then only meet every other tile, and
      * the faster ones do not stand at a barrier while the slower ones finish every single tile. */
-    constexpr int GROUP = WAVES == 8 ? 2 : 1;
+    constexpr int GROUP = WAVES * NB >= 12 ? 2 : 1;
     constexpr int NSTAGE = 2 * GROUP;                    /* the group in use and the group on its way */
 
     /* XCD-aware numbering: hardware deals workgroups round-robin to the 8
@@ -331,25 +339,19 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     const int head = work / q_tiles;
     int qt = work - head * q_tiles;
     if (CAUSAL) qt = q_tiles - 1 - qt;             /* longest rows first */
+    const int q0 = qt * BM;
     const int kvh = head / kv_group;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;       /* 16x16 block: column li, row group lg */
-    const int q0 = qt * BM, wq0 = q0 + wave * 32;
-    const int qrow0 = wq0 + li, qrow1 = qrow0 + 16; /* this lane's two queries (query blocks 0 and 1) */
+    const int wq0 = q0 + wave * WQ;
+    const int qrow0 = wq0 + li;                     /* this lane's queries: qrow0 + 16 nb, one per query block */
 
     const uint16_t *kbase = k + (size_t)kvh * HD;
     const uint16_t *vbase = v + (size_t)kvh * HD;
 
-    f32x4 o[8][2];                                   /* O^T: dims 16db + 4lg + r of query block nb */
-#pragma unroll
-    for (int db = 0; db < 8; db++)
-#pragma unroll
-        for (int nb = 0; nb < 2; nb++) o[db][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    float m_run[2] = {-INFINITY, -INFINITY};
     /* row sums on the matrix cores: an all-ones A operand makes every row of the product the
      * column sum of P^T, i.e. the sum of the lane's query over the tile's keys */
-    f32x4 l_acc[2] = {f32x4{0.0f, 0.0f, 0.0f, 0.0f}, f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
     const bf16x8 ones = __builtin_bit_cast(bf16x8, u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
 
     int k_end = seq_k;
@@ -372,18 +374,10 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     }
 
     /* This lane's source offsets inside a piece (bytes): row lane/16 of the piece, chunk by parity of the piece. */
-    const int last_k0 = (ntiles - 1) * BN;
     uint32_t lane_off[2];
 #pragma unroll
     for (int par = 0; par < 2; par++)
         lane_off[par] = (uint32_t)((lane >> 4) * ldi + 8 * ((lane & 15) ^ swz(4 * par + (lane >> 4)))) * 2u;
-    auto request = [&](int tile_index, int stage) {      /* tile indices past the end repeat the last tile */
-        const int kn = min(tile_index * BN, last_k0);
-        const uint16_t *kt = kbase + (size_t)kn * ldi, *vt = vbase + (size_t)kn * ldi;
-        if (kn + BN <= seq_k) load_tile<NI>(lds + stage * STAGE, kt, vt, ldi, lane_off, wave);
-        else load_tile_clamped<NI>(lds + stage * STAGE, kt, vt, ldi, seq_k - 1 - kn, lane, wave);
-    };
-
     /* The key mask as one 64-bit word per key tile, kept in LDS behind the stages: built once here,
      * so that the loop has no global load of its own (a load there would be waited for with
      * vmcnt(0), i.e. together with the newest tile requests). Keys past seq_k count as masked. */
@@ -396,15 +390,34 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         }
     }
 
+    const int last_k0 = (ntiles - 1) * BN;
+    auto request = [&](int tile_index, int stage) {      /* tile indices past the end repeat the last tile */
+        const int kn = min(tile_index * BN, last_k0);
+        const uint16_t *kt = kbase + (size_t)kn * ldi, *vt = vbase + (size_t)kn * ldi;
+        if (kn + BN <= seq_k) load_tile<NI, WAVES>(lds + stage * STAGE, kt, vt, ldi, lane_off, wave);
+        else load_tile_clamped<NI, WAVES>(lds + stage * STAGE, kt, vt, ldi, seq_k - 1 - kn, lane, wave);
+    };
+
+    f32x4 o[8][NB];                                  /* O^T: dims 16db + 4lg + r of query block nb */
+    float m_run[NB], neg_m[NB], bound[NB];           /* running max; its negative (0 while it is -inf); (max + margin) / scale */
+    f32x4 l_acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+#pragma unroll
+        for (int db = 0; db < 8; db++) o[db][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        m_run[nb] = -INFINITY; neg_m[nb] = 0.0f; bound[nb] = -INFINITY;
+        l_acc[nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    const float inv_scale_log2 = 1.0f / scale_log2;
     /* ---- prologue: the first group of tiles is requested before Q, so that the two fetches overlap ---- */
 #pragma unroll
     for (int t = 0; t < GROUP; t++) request(t, t);
 
     /* Q^T as B operands: for query block nb and k-step ks the lane holds dims 32ks + 8lg .. +7
      * of query 16nb + li. */
-    bf16x8 qb[2][4];
+    bf16x8 qb[NB][4];
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
+    for (int nb = 0; nb < NB; nb++) {
         const uint16_t *qp = q + (size_t)min(qrow0 + 16 * nb, seq_q - 1) * ldi + (size_t)head * HD + 8 * lg;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++)
@@ -412,7 +425,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     }
     if (qnorm.w) {                                   /* wave-uniform */
 #pragma unroll
-        for (int nb = 0; nb < 2; nb++) norm_rope_q_fragment(qb[nb], qnorm, min(qrow0 + 16 * nb, seq_q - 1), lg);
+        for (int nb = 0; nb < NB; nb++) norm_rope_q_fragment(qb[nb], qnorm, min(qrow0 + 16 * nb, seq_q - 1), lg);
     }
 
     /* The tile requests are invisible to the compiler's own wait-count bookkeeping, so every load it
@@ -422,7 +435,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
      * compiler sinks the Q loads to the loop and re-waits for them in every iteration, which in fact
      * waits for the newest tile requests. */
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++)
+    for (int nb = 0; nb < NB; nb++)
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
             u32x4 t = __builtin_bit_cast(u32x4, qb[nb][ks]);
@@ -453,7 +466,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
          * LDS before the eight MFMAs of step ks are issued, so that the LDS serves reads all the
          * time the matrix core works instead of in one burst from all waves that the MFMAs then
          * wait for. Each operand feeds two MFMAs. ---- */
-        f32x4 s[4][2];
+        f32x4 s[4][NB];
         {
             u32x4 ka[2][4];                                /* two k-steps in flight */
             auto read_k = [&](int ks) {
@@ -472,7 +485,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 #pragma unroll
                 for (int mb = 0; mb < 4; mb++)
 #pragma unroll
-                    for (int nb = 0; nb < 2; nb++)
+                    for (int nb = 0; nb < NB; nb++)
                         s[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[ks & 1][mb]), qb[nb][ks],
                                                                             ks == 0 ? zero : s[mb][nb], 0, 0, 0);
                 
@@ -498,39 +511,63 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             for (int mb = 0; mb < 4; mb++)
 #pragma unroll
                 for (int r = 0; r < 4; r++)
-                    if (!((mine >> (16 * mb + r)) & 1ull)) { s[mb][0][r] = -INFINITY; s[mb][1][r] = -INFINITY; }
+                    if (!((mine >> (16 * mb + r)) & 1ull)) {
+#pragma unroll
+                        for (int nb = 0; nb < NB; nb++) s[mb][nb][r] = -INFINITY;
+                    }
         }
         if (CAUSAL && k0 + BN - 1 > wq0) {
             const int lim0 = qrow0 - k0 - 4 * lg;      /* key offset 16mb + r valid iff <= lim */
 #pragma unroll
             for (int mb = 0; mb < 4; mb++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    if (16 * mb + r > lim0) s[mb][0][r] = -INFINITY;
-                    if (16 * mb + r > lim0 + 16) s[mb][1][r] = -INFINITY;
-                }
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++)
+                        if (16 * mb + r > lim0 + 16 * nb) s[mb][nb][r] = -INFINITY;
         }
 
         /* ---- online softmax: the lane holds 16 of the 64 scores of each of its two queries;
-         * the other three quarters sit in the lanes 16, 32 and 48 away ---- */
-        float mx[2];
+         * the other three quarters sit in the lanes 16, 32 and 48 away.
+         * The running max is only raised when some score of the wave exceeds it by more than
+         * 2^8, and that test needs no cross-lane traffic: "the largest of a query's 64 scores
+         * exceeds the bound" is the same as "the largest of the 16 that some lane holds does",
+         * because the four lanes of a query share the bound. So the common tile pays for the
+         * per-lane maxima and one compare per query block, and only a tile that does raise the
+         * max (the first few of a row) combines the four lanes and rescales. The bound is kept
+         * in score units (bound[nb] = (m_run[nb] + 2^8 margin) / scale), next to -m_run. ---- */
+        float lane_max[NB];
+        bool raise = false;
+        {
+            float t[NB][6];
 #pragma unroll
-        for (int nb = 0; nb < 2; nb++) {
-            const float t1 = max3(s[0][nb][0], s[0][nb][1], s[0][nb][2]);
-            const float t2 = max3(s[0][nb][3], s[1][nb][0], s[1][nb][1]);
-            const float t3 = max3(s[1][nb][2], s[1][nb][3], s[2][nb][0]);
-            const float t4 = max3(s[2][nb][1], s[2][nb][2], s[2][nb][3]);
-            const float t5 = max3(s[3][nb][0], s[3][nb][1], s[3][nb][2]);
-            const float u1 = max3(t1, t2, t3), u2 = max3(t4, t5, s[3][nb][3]);
-            mx[nb] = quad_group_max(max3(u1, u2, u2)) * scale_log2;
+            for (int nb = 0; nb < NB; nb++) {                  /* independent chains, written side by side */
+                t[nb][0] = max3(s[0][nb][0], s[0][nb][1], s[0][nb][2]);
+                t[nb][1] = max3(s[0][nb][3], s[1][nb][0], s[1][nb][1]);
+                t[nb][2] = max3(s[1][nb][2], s[1][nb][3], s[2][nb][0]);
+                t[nb][3] = max3(s[2][nb][1], s[2][nb][2], s[2][nb][3]);
+                t[nb][4] = max3(s[3][nb][0], s[3][nb][1], s[3][nb][2]);
+            }
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                t[nb][0] = max3(t[nb][0], t[nb][1], t[nb][2]);
+                t[nb][5] = max3(t[nb][3], t[nb][4], s[3][nb][3]);
+            }
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                lane_max[nb] = fmaxf(t[nb][0], t[nb][5]);
+                raise = raise || lane_max[nb] > bound[nb];
+            }
         }
 
-        if (__any(mx[0] > m_run[0] + RESCALE_THRESHOLD || mx[1] > m_run[1] + RESCALE_THRESHOLD)) {
+        if (__any(raise)) {
 #pragma unroll
-            for (int nb = 0; nb < 2; nb++) {
-                const float m_new = fmaxf(m_run[nb], mx[nb]);
+            for (int nb = 0; nb < NB; nb++) {
+                const float m_new = fmaxf(m_run[nb], quad_group_max(lane_max[nb]) * scale_log2);
                 const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - (m_new == -INFINITY ? 0.0f : m_new));
                 m_run[nb] = m_new;
+                neg_m[nb] = m_new == -INFINITY ? 0.0f : -m_new;     /* finite while every key so far is masked */
+                bound[nb] = (m_new + RESCALE_THRESHOLD) * inv_scale_log2;
                 l_acc[nb] *= alpha;
 #pragma unroll
                 for (int db = 0; db < 8; db++) o[db][nb] *= alpha;
@@ -539,17 +576,16 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 
         /* P^T as B operands: k-step ks covers keys 32ks .. 32ks+31, of which this lane's 8 are
          * 32ks + 4lg + r (key block 2ks) and 32ks + 16 + 4lg + r (key block 2ks+1). */
-        u32x4 pw[2][2];
+        u32x4 pw[2][NB];
 #pragma unroll
-        for (int nb = 0; nb < 2; nb++) {
-            const float neg_m = m_run[nb] == -INFINITY ? 0.0f : -m_run[nb];   /* finite while every key so far is masked */
+        for (int nb = 0; nb < NB; nb++) {
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
                 float p[8];
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    p[r] = __builtin_amdgcn_exp2f(fmaf(s[2 * ks][nb][r], scale_log2, neg_m));
-                    p[4 + r] = __builtin_amdgcn_exp2f(fmaf(s[2 * ks + 1][nb][r], scale_log2, neg_m));
+                    p[r] = __builtin_amdgcn_exp2f(fmaf(s[2 * ks][nb][r], scale_log2, neg_m[nb]));
+                    p[4 + r] = __builtin_amdgcn_exp2f(fmaf(s[2 * ks + 1][nb][r], scale_log2, neg_m[nb]));
                 }
                 pw[ks][nb] = u32x4{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
             }
@@ -576,17 +612,19 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                 __builtin_amdgcn_sched_barrier(0);
                 
                 const int ks = g >> 1;
-                const bf16x8 pb0 = __builtin_bit_cast(bf16x8, pw[ks][0]), pb1 = __builtin_bit_cast(bf16x8, pw[ks][1]);
                 if ((g & 1) == 0) {
-                    l_acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb0, l_acc[0], 0, 0, 0);
-                    l_acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb1, l_acc[1], 0, 0, 0);
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++)
+                        l_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, __builtin_bit_cast(bf16x8, pw[ks][nb]), l_acc[nb], 0, 0, 0);
                 }
 #pragma unroll
                 for (int d = 0; d < 4; d++) {
                     const int db = 4 * (g & 1) + d;
                     s16x8 both = __builtin_shufflevector(lo[g & 1][d], hi[g & 1][d], 0, 1, 2, 3, 4, 5, 6, 7);
-                    o[db][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb0, o[db][0], 0, 0, 0);
-                    o[db][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb1, o[db][1], 0, 0, 0);
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++)
+                        o[db][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), __builtin_bit_cast(bf16x8, pw[ks][nb]),
+                                                                            o[db][nb], 0, 0, 0);
                 }
                 
                 __builtin_amdgcn_sched_barrier(0);
@@ -601,9 +639,9 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 
     wait_vmcnt<0>();       /* nothing may still be on its way into the LDS when it is given back (the loop ends with this wait too) */
 
-    /* ---- normalise and store: the lane holds dims 16db + 4lg + {0..3} of its two queries ---- */
+    /* ---- normalise and store: the lane holds dims 16db + 4lg + {0..3} of its queries ---- */
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
+    for (int nb = 0; nb < NB; nb++) {
         const float l_tot = l_acc[nb][0];              /* every row of the ones product is the full sum */
         const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
         const int qrow = qrow0 + 16 * nb;
@@ -620,43 +658,43 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     }
 }
 
-template <int W> constexpr size_t stage_bytes() { return (W == 8 ? 4 : 2) * STAGE * sizeof(uint16_t); }
+template <int W, int NB> constexpr size_t stage_bytes() { return (W * NB >= 12 ? 4 : 2) * STAGE * sizeof(uint16_t); }
 constexpr size_t LDS_MAX = 160 * 1024;
 constexpr int CUS = 256;
 
-template <int W, bool C, bool M>
+template <int W, int NB, bool C, bool M>
 int launch(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
            const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads,
            float scale, const int *key_mask, const QNorm &qn) {
     static bool configured = false;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd128<W, C, M>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd128<W, NB, C, M>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
         if (e != hipSuccess) return (int)e;
         configured = true;
     }
-    const int q_tiles = (seq_q + 32 * W - 1) / (32 * W);
+    const int q_tiles = (seq_q + 16 * NB * W - 1) / (16 * NB * W);
     const int total = q_tiles * heads;
     const int per_xcd = (total + XCDS - 1) / XCDS;
     /* the stages, and for a key mask one 64-bit word per key tile behind them */
-    const size_t lds_bytes = stage_bytes<W>() + (M ? 8 * (size_t)((seq_k + BN - 1) / BN) : 0);
+    const size_t lds_bytes = stage_bytes<W, NB>() + (M ? 8 * (size_t)((seq_k + BN - 1) / BN) : 0);
     if (lds_bytes > LDS_MAX) return (int)hipErrorInvalidValue;       /* the caller keeps masked seq_k below the limit */
-    hipLaunchKernelGGL((k_fa_fwd_hd128<W, C, M>), dim3(per_xcd * XCDS), dim3(64 * W), lds_bytes, st, out, ldo,
+    hipLaunchKernelGGL((k_fa_fwd_hd128<W, NB, C, M>), dim3(per_xcd * XCDS), dim3(64 * W), lds_bytes, st, out, ldo,
                        q, k, v, ldi, seq_q, seq_k, q_tiles, total, per_xcd, heads / kv_heads,
                        scale * 1.4426950408889634f, key_mask, qn);
     return (int)hipGetLastError();
 }
 
-template <int W>
+template <int W, int NB = 2>
 int launch_w(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
              const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads, float scale,
              int causal, const int *key_mask, const QNorm &qn) {
     if (causal) {
-        if (key_mask) return launch<W, true, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
-        return launch<W, true, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
+        if (key_mask) return launch<W, NB, true, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
+        return launch<W, NB, true, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
     }
-    if (key_mask) return launch<W, false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
-    return launch<W, false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
+    if (key_mask) return launch<W, NB, false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
+    return launch<W, NB, false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
 }
 
 }  // namespace
