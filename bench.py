@@ -42,9 +42,21 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 matrix peak (vendor figure)
 PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E peak
-# HBM bytes one C2 attention launch moves, from the FETCH_SIZE and WRITE_SIZE hardware counters scaled by a
-# 1 GiB copy kernel (profiles/k_fa_fwd_hd128__c2__hbm_traffic.txt): 103.9 MB read + 28.3 MB written.
-C2_ATTENTION_HBM_TRAFFIC = 132_277_000
+# HBM bytes one C2 attention launch moves come from hardware counters (FETCH_SIZE, WRITE_SIZE scaled by a 1 GiB
+# copy kernel), which a separate profiler run collects: the summary of that run is read here, so the figure in the
+# output line is the one on file and says so.
+TRAFFIC_PROFILE = os.path.join("profiles", "k_fa_fwd_hd128__c2__hbm_traffic.txt")
+
+
+def traffic_on_file():
+    """(bytes per launch, source) from the line 'total_bytes_per_launch: N' of the committed counter summary."""
+    try:
+        for line in open(os.path.join(ROOT, TRAFFIC_PROFILE)):
+            if line.startswith("total_bytes_per_launch:"):
+                return int(line.split(":")[1].strip().replace(",", "")), TRAFFIC_PROFILE
+    except OSError:
+        pass
+    return None, None
 
 _vp = C.c_void_p
 
@@ -212,6 +224,18 @@ def event_time(hip, stream, fn, reps, start=0):
     return hip.elapsed_ms(a, b) / reps
 
 
+def single_launch_ms(hip, stream, lib, fn, reps=5):
+    """One launch on an idle stream, events around it: what a caller that waits for the result sees
+    beyond the kernel itself (median of `reps`)."""
+    ts = []
+    for i in range(reps):
+        lib.iris_dev_sync()
+        a, b = hip.event(), hip.event()
+        hip.record(a, stream); fn(i); hip.record(b, stream)
+        ts.append(hip.elapsed_ms(a, b))
+    return float(np.median(ts))
+
+
 def per_launch_times(hip, stream, fn, reps, before=None):
     """Per-launch ms with an event pair around every launch (for kernels >> event cost); `before(i)`, if given,
     is enqueued ahead of each timed launch, outside its event pair."""
@@ -318,6 +342,65 @@ def microbench_lib():
     mb.iris_mb_copy.argtypes = [_vp, _vp, _vp, C.c_size_t]
     mb.iris_mb_rmw.argtypes = [_vp, _vp, C.c_size_t]
     return mb
+
+
+def vae_case(rng, seq=16384):
+    """The VAE mid-block attention of a 1024 x 1024 image: one head of 512 over (1024 / 8)^2 tokens, rows q | k | v."""
+    hd = 512
+    c = dict(name="VAE", hd=hd, causal=False, key_mask=None, heads=1, kv_heads=1, seq=seq, q_dim=hd, kv_dim=hd,
+             ldi=3 * hd, ldo=hd, scale=float(1.0 / np.sqrt(np.float32(hd))))
+    c["buf"] = to_bf16(rng.standard_normal((seq, 3 * hd), dtype=np.float32))
+    return c
+
+
+def only_one(dev, hip, stream, rng, name, steps, settle_ms):
+    """Launches of one configuration only (for profiler runs)."""
+    lib = dev.lib
+    if name == "VAE":
+        c = vae_case(rng)
+        d, o = dev.to_device(c["buf"]), lib.iris_dev_alloc(c["seq"] * c["ldo"] * 2)
+        fn = lambda i: lib.iris_dev_attention(o, c["ldo"], d, _vp(d + 2 * c["q_dim"]), _vp(d + 2 * (c["q_dim"] + c["kv_dim"])),
+                                              c["ldi"], c["seq"], c["seq"], 1, 1, c["hd"], c["scale"], 0, None)
+        settle(lib, fn, settle_ms)
+        ts = per_launch_times(hip, stream, fn, steps)
+        dev.check()
+        kernel = dev.last_kernel()
+        lib.iris_dev_free(d); lib.iris_dev_free(o)
+    else:
+        c = make_config(name, rng)
+        r = Resident(dev, c, 2)
+        settle(lib, r.step, settle_ms)
+        ts = per_launch_times(hip, stream, r.attention, steps, before=lambda i: (r.norm_q(i), r.norm_k(i)))
+        dev.check()
+        kernel = dev.last_kernel()
+        r.free()
+    fl = attention_flops(c)
+    return {"config": name, "kernel": kernel, "launches": steps, "attention_ms_mean": round(float(np.mean(ts)), 4),
+            "attention_ms_median": round(float(np.median(ts)), 4), "attention_ms_min": round(float(np.min(ts)), 4),
+            "flops_per_launch": fl, "tflops": round(fl / float(np.mean(ts)) / 1e9, 1)}
+
+
+def occupancy_probe(dev, hip, stream, rng, settle_ms):
+    """The attention kernel on one round of workgroups that fills all 256 CUs, 176 of them and 128 of them
+    (4096 tokens x 16 / 11 / 8 heads: 256 / 176 / 128 workgroups of 256 queries, each walking the same 64 key
+    tiles). The schedule of a workgroup is the same in all three; what changes is how many CUs draw power."""
+    lib, res = dev.lib, []
+    for heads in (16, 11, 8):
+        c = dict(name=f"{heads}h", hd=128, causal=False, key_mask=None, heads=heads, kv_heads=heads, seq=4096,
+                 q_dim=heads * 128, kv_dim=heads * 128, ldi=3 * heads * 128, ldo=heads * 128,
+                 scale=float(1.0 / np.sqrt(np.float32(128))))
+        c["buf"] = to_bf16(rng.standard_normal((4096, c["ldi"]), dtype=np.float32))
+        d, o = dev.to_device(c["buf"]), lib.iris_dev_alloc(4096 * c["ldo"] * 2)
+        fn = lambda i: lib.iris_dev_attention(o, c["ldo"], d, _vp(d + 2 * c["q_dim"]), _vp(d + 2 * (c["q_dim"] + c["kv_dim"])),
+                                              c["ldi"], 4096, 4096, heads, heads, 128, c["scale"], 0, None)
+        settle(lib, fn, settle_ms)
+        ms = float(np.median(per_launch_times(hip, stream, fn, 30)))
+        dev.check()
+        fl = attention_flops(c)
+        res.append({"workgroups": heads * 16, "launch_us": round(ms * 1e3, 1), "tflops": round(fl / ms / 1e9, 1),
+                    "tflops_per_busy_cu": round(fl / ms / 1e9 / min(heads * 16, 256), 3)})
+        lib.iris_dev_free(d); lib.iris_dev_free(o)
+    return res
 
 
 def copy_only(dev, hip, stream, nbytes, reps):
@@ -436,6 +519,28 @@ def cpu_baseline(c):
             "rope_tables_ms": round(dtab * 1e3, 2)}
 
 
+def cpu_seconds(c, calls=1):
+    """Seconds per attention call of the reference's BLAS-build CPU structure on this host for configuration c
+    (f32; 256-query chunks where the full score matrix would not fit, as the reference's FLUX.3 path does)."""
+    import oracle
+    base = oracle.cpu_baseline()
+    f = (c["buf"].astype(np.uint32) << 16).view(np.float32)
+    q = np.ascontiguousarray(f[:, :c["q_dim"]])
+    k = np.ascontiguousarray(f[:, c["q_dim"]:c["q_dim"] + c["kv_dim"]])
+    v = np.ascontiguousarray(f[:, c["q_dim"] + c["kv_dim"]:])
+    cores = base.online_cpus()
+    box_share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    limit = min(cores, box_share) if box_share > 0 else cores
+    chunk = 256 if c["seq"] > 6000 else 0
+    times, threads = [], 0
+    for _ in range(calls + 1):
+        t0 = time.perf_counter()
+        _, threads = base.attention(q, k, v, c["heads"], c["kv_heads"], c["scale"], c["causal"], c["key_mask"],
+                                    q_chunk=chunk, threads=limit)
+        times.append(time.perf_counter() - t0)
+    return float(np.mean(times[1:])), threads, chunk
+
+
 # ----------------------------------------------------------------------------- main
 def main():
     ap = argparse.ArgumentParser()
@@ -451,6 +556,10 @@ def main():
     ap.add_argument("--no-variants", action="store_true",
                     help="skip the two alternative forms of the step (fused Q+K norm, Q norm inside attention), so that "
                          "a profile of the run holds the launches of the reference's call pattern only")
+    ap.add_argument("--only", default="", metavar="CONFIG",
+                    help="only launch one configuration's kernels, --steps times each, after the settling load: "
+                         "C1, C2, C3-cond, C3-uncond, C4, C5 (norm+rope on Q, on K, attention) or VAE (the 512-wide "
+                         "single head over 16384 tokens). For profiler runs of the other configurations.")
     ap.add_argument("--copy-only", type=int, default=0, metavar="MiB",
                     help="only launch the plain copy kernel on MiB of data, --steps times (the known-size "
                          "launch that hardware byte counters are scaled by)")
@@ -466,6 +575,10 @@ def main():
     rng = np.random.default_rng(20250101)
     if args.copy_only:
         print(json.dumps(copy_only(dev, hip, stream, args.copy_only << 20, args.steps)))
+        return
+
+    if args.only:
+        print(json.dumps(only_one(dev, hip, stream, rng, args.only, args.steps, args.settle_ms)))
         return
 
     c2 = make_config("C2", rng)
@@ -512,6 +625,8 @@ def main():
     att = per_launch_times(hip, stream, res.attention, max(args.steps, 10),
                            before=lambda i: (res.norm_q(i), res.norm_k(i)))
     att_ms = float(np.mean(att))
+    att_single = single_launch_ms(hip, stream, lib, res.attention)
+    traffic, traffic_source = traffic_on_file()
     # bandwidth-bound kernel: back-to-back launches over rotating buffers (cold) and one buffer (warm)
     reps = max(args.steps, 2 * copies)
     nr_q_ms = event_time(hip, stream, res.norm_q, reps)
@@ -523,6 +638,7 @@ def main():
 
     out = {
         "metric": "joint_attention_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+        "value_from_idle": round(flops / (idle_ms * 1e-3) / 1e12, 2),
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_steps": settle_steps,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -540,8 +656,11 @@ def main():
             "note": "two launches: iris_dev_head_norm_rope on K + iris_dev_attention_qnorm"},
         "roofline": {"kernel": "k_fa_fwd_hd128", "bound": "mfma", "achieved": round(flops / (att_ms * 1e-3) / 1e12, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / (att_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
-                     "traffic": C2_ATTENTION_HBM_TRAFFIC, "traffic_unit": "bytes per launch (hardware counters, profiled separately)",
-                     "algorithmic_bytes": 4 * c2["seq"] * c2["q_dim"] * 2, "launch_ms": round(att_ms, 4), "launch_ms_min": round(float(np.min(att)), 4),
+                     "traffic": traffic, "traffic_unit": "bytes per launch, hardware counters of a separate profiler run",
+                     "traffic_source": traffic_source,
+                     "algorithmic_bytes": 4 * c2["seq"] * c2["q_dim"] * 2, "launch_ms": round(att_ms, 4),
+                     "launch_ms_median": round(float(np.median(att)), 4), "launch_ms_min": round(float(np.min(att)), 4),
+                     "single_launch_ms": round(att_single, 4),
                      "flops_per_launch": flops},
         "norm_rope": {"kernel": "k_norm_rope_hd128", "bound": "hbm", "unit": "GB/s", "peak": PEAK_HBM_GBPS,
                       "bytes_per_call": q_bytes,
@@ -550,7 +669,12 @@ def main():
                       "qk_fused_us": round(nr_qk_ms * 1e3, 2), "qk_fused_gbps": round(qk_bytes / (nr_qk_ms * 1e-3) / 1e9, 1),
                       "qk_fused_frac": round(qk_bytes / (nr_qk_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
                       "warm_cache_q_call_us": round(nr_warm_ms * 1e3, 2),
-                      "note": "cold = 8 rotating 85 MB row buffers (> 256 MB Infinity Cache); warm = same buffer every call"},
+                      "warm_cache_q_call_frac": round(q_bytes / (nr_warm_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                      "q_call_single_launch_us": round(single_launch_ms(hip, stream, lib, res.norm_q) * 1e3, 2),
+                      "note": "cold = 8 rotating 85 MB row buffers (> 256 MB Infinity Cache); warm = same buffer every call; "
+                              "averages over back-to-back launches between two events. In a kernel trace of the same series "
+                              "consecutive launches abut, so these are also the kernel-only durations "
+                              "(profiles/k_norm_rope_hd128__c2__kernel_trace.txt)"},
     }
     res.free()
 
@@ -558,21 +682,36 @@ def main():
         shapes = []
         for name in ("C1", "C2", "C3-cond", "C3-uncond", "C4", "C5"):
             c = c2 if name == "C2" else make_config(name, rng)
-            r = Resident(dev, c, 2)
+            # enough rotating row buffers that the norm+rope reads come from HBM (> 2 x the 256 MB Infinity Cache)
+            r = Resident(dev, c, int(min(64, max(2, np.ceil(600e6 / c["buf"].nbytes)))))
             for i in range(3):
                 r.step(i)
             settle(lib, r.attention, args.settle_ms / 2)
             n = 20
-            a_ms = float(np.mean(per_launch_times(hip, stream, r.attention, n)))
-            qk_ms = event_time(hip, stream, r.norm_qk, n)
+            a = per_launch_times(hip, stream, r.attention, n)
+            a_ms = float(np.mean(a))
+            q_ms = event_time(hip, stream, r.norm_q, 2 * n)
+            qk_ms = event_time(hip, stream, r.norm_qk, 2 * n)
             fl = attention_flops(c)
-            nb = norm_rope_bytes(c["seq"], c["heads"]) + norm_rope_bytes(c["seq"], c["kv_heads"])
-            shapes.append({"config": name, "seq": c["seq"], "heads": c["heads"], "kv_heads": c["kv_heads"],
-                           "attention_ms": round(a_ms, 4), "attention_tflops": round(fl / a_ms / 1e9, 2),
-                           "attention_frac_of_mfma_peak": round(fl / a_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
-                           "norm_rope_qk_us": round(qk_ms * 1e3, 2), "norm_rope_qk_gbps": round(nb / qk_ms / 1e6, 1)})
+            qb = norm_rope_bytes(c["seq"], c["heads"])
+            nb = qb + norm_rope_bytes(c["seq"], c["kv_heads"])
+            entry = {"config": name, "seq": c["seq"], "heads": c["heads"], "kv_heads": c["kv_heads"],
+                     "attention_ms": round(a_ms, 4), "attention_ms_median": round(float(np.median(a)), 4),
+                     "attention_ms_min": round(float(np.min(a)), 4),
+                     "attention_single_launch_ms": round(single_launch_ms(hip, stream, lib, r.attention), 4),
+                     "attention_tflops": round(fl / a_ms / 1e9, 2),
+                     "attention_frac_of_mfma_peak": round(fl / a_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                     "norm_rope_q_us": round(q_ms * 1e3, 2), "norm_rope_q_gbps": round(qb / q_ms / 1e6, 1),
+                     "norm_rope_q_frac_of_hbm_peak": round(qb / q_ms / 1e6 / PEAK_HBM_GBPS, 4),
+                     "norm_rope_qk_us": round(qk_ms * 1e3, 2), "norm_rope_qk_gbps": round(nb / qk_ms / 1e6, 1),
+                     "norm_rope_qk_frac_of_hbm_peak": round(nb / qk_ms / 1e6 / PEAK_HBM_GBPS, 4)}
             dev.check()
             r.free()
+            if not args.no_cpu:
+                secs, threads, chunk = cpu_seconds(c)
+                entry.update(cpu_seconds=round(secs, 4), cpu_tflops=round(fl / secs / 1e12, 4), cpu_threads=threads,
+                             cpu_query_chunk=chunk)
+            shapes.append(entry)
         out["shapes"] = shapes
 
     if not args.no_shapes:
@@ -580,6 +719,7 @@ def main():
         out["rope_tables"] = rope_table_times(dev, c2)
     if not args.no_machine:
         out["machine"] = machine_ceilings(dev, hip, stream)
+        out["machine"]["attention_by_busy_cus"] = occupancy_probe(dev, hip, stream, rng, args.settle_ms / 3)
         # The ABI takes device pointers, so `value` has no host transfer in it. For a caller that had the
         # fused qkv rows in host memory, this is the rate with the upload of those rows counted.
         row_bytes = c2["buf"].nbytes
