@@ -62,7 +62,18 @@ void iris_dev_head_norm_rope(uint16_t *x, int ld, const float *w,
  * heads (GQA), query head h uses kv head h / (heads / kv_heads).
  * causal: query i ignores keys j > i. key_mask: device int [seq_k],
  * 0 = ignored key, or NULL. A query with no valid key gives a zero row
- * (reference iris_cuda.cu:531, 650, 676). */
+ * (reference iris_cuda.cu:531, 650, 676).
+ * Every combination of heads / kv_heads / head_dim / stride / alignment is answered, as in the
+ * reference, with one limit: head_dim <= 2048 (larger is reported as an error; the reference's
+ * GEMM-based fallback has no such limit, none of its models comes near it). head_dim 128, 256
+ * and 512 on 16-byte aligned rows run on the matrix cores directly, any other head_dim <= 512 or
+ * alignment through a padded, aligned private copy of q, k, v; the rest (head_dim > 512,
+ * scale <= 0, more than 250000 masked keys) on a scalar kernel.
+ * Numerics: P = exp(s - max) is rounded to bf16 for the P V product, as in the reference's GPU
+ * kernels (iris_cuda.cu:656-665), and the row sum in the denominator is taken over those ROUNDED
+ * values (on the matrix cores), where the reference sums the unrounded f32 values (:659-665): the
+ * output weights then add up to exactly one; the two differ by the mean bf16 rounding error of a
+ * row, far inside the tolerance against the fp32 CPU attention. */
 void iris_dev_attention(uint16_t *out, int ldo,
                         const uint16_t *q, const uint16_t *k, const uint16_t *v,
                         int ldi, int seq_q, int seq_k, int heads, int kv_heads,

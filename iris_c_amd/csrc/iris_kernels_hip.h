@@ -56,12 +56,24 @@ int iris_hip_fa_sliced(void *stream, uint16_t *out, int ldo, const uint16_t *q,
                        int heads, int kv_heads, int head_dim, float scale, int causal,
                        const int *key_mask);
 
-/* Any head_dim <= 512, any stride / alignment / scale; the rows of q may have a stride (ldq) of
- * their own. Correctness path. */
+/* Any head_dim <= IRIS_ATTENTION_MAX_HEAD_DIM (the 8 queries of a workgroup are kept in LDS as f32),
+ * any stride / alignment / scale; the rows of q may have a stride (ldq) of their own. Correctness path. */
+#define IRIS_ATTENTION_MAX_HEAD_DIM 2048
 int iris_hip_attention_generic(void *stream, uint16_t *out, int ldo, const uint16_t *q, int ldq,
                                const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
                                int seq_k, int heads, int kv_heads, int head_dim, float scale,
                                int causal, const int *key_mask);
+
+/* Padded, aligned copy of q, k, v for the matrix-core kernels: dst is one fused row buffer
+ * [max(seq_q, seq_k)][(heads + 2 kv_heads) * hdp] (q | k | v), 16-byte aligned, every head's hd
+ * elements followed by hdp - hd zeros (hdp a multiple of 8, >= hd); rows a tensor does not have are
+ * zero. Sources: any stride and alignment. unpack copies the first hd of every hdp output columns
+ * back into rows of any stride and alignment. */
+int iris_hip_pack_heads(void *stream, uint16_t *dst, const uint16_t *q, int ldq, int seq_q,
+                        const uint16_t *k, const uint16_t *v, int ldkv, int seq_k,
+                        int heads, int kv_heads, int hd, int hdp);
+int iris_hip_unpack_heads(void *stream, uint16_t *out, int ldo, const uint16_t *src, int ld_src,
+                          int rows, int heads, int hd, int hdp);
 
 /* ---- elementwise and normalisation operators (ew_norm_ops.hip): any size and alignment,
  * 16-byte accesses when the pointers and sizes allow ---- */

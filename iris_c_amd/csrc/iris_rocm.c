@@ -36,6 +36,9 @@ static size_t g_gn_scratch_floats = 0;
 /* normalised copy of Q for the iris_dev_attention_qnorm calls that the matrix-core kernel does not take */
 static uint16_t *g_q_scratch = NULL;
 static size_t g_q_scratch_bytes = 0;
+/* padded, aligned copy of q | k | v (and the padded output) for attention calls on other head sizes or alignments */
+static uint16_t *g_pack = NULL;
+static size_t g_pack_bytes = 0;
 /* staging buffer of the rotary tables being expanded: column map, row offsets, dictionary */
 static void *g_rope_stage = NULL;
 static size_t g_rope_stage_bytes = 0;
@@ -99,6 +102,9 @@ void iris_dev_cleanup(void) {
     if (g_gn_scratch) check(hipFree(g_gn_scratch), "free");
     if (g_rope_stage) check(hipFree(g_rope_stage), "free");
     if (g_q_scratch) check(hipFree(g_q_scratch), "free");
+    if (g_pack) check(hipFree(g_pack), "free");
+    g_pack = NULL;
+    g_pack_bytes = 0;
     g_q_scratch = NULL;
     g_q_scratch_bytes = 0;
     iris_lt_release();
@@ -155,6 +161,26 @@ void iris_dev_sync(void) {
 
 static int aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
+/* Private scratch that only grows: makes *p hold at least `need` bytes (the old block is released once the
+ * work that may still read it has drained). Returns 0 after reporting a failed allocation. */
+static int scratch_fit(void **p, size_t *have, size_t need, const char *what) {
+    if (need <= *have) return 1;
+    if (*p) {
+        check(hipStreamSynchronize(g_stream), "sync");
+        check(hipFree(*p), "free");
+    }
+    *p = NULL;
+    *have = 0;
+    if (hipMalloc(p, need) != hipSuccess) {
+        (void)hipGetLastError();
+        *p = NULL;
+        fail(-1, what, "scratch allocation failed");
+        return 0;
+    }
+    *have = need;
+    return 1;
+}
+
 /* Shared by the one- and two-tensor entries; xk may be NULL with k_heads 0. */
 static void norm_rope(uint16_t *xq, uint16_t *xk, int ld, const float *wq, const float *wk,
                       const float *rope_cos, const float *rope_sin, int seq, int q_heads,
@@ -209,8 +235,8 @@ static void attention(const char *what, uint16_t *out, int ldo,
                       float eps, int split_half) {
     if (!need_ready(what)) return;
     if (seq_q <= 0 || heads <= 0) return;
-    if (kv_heads <= 0 || heads % kv_heads != 0 || head_dim <= 0 || head_dim > 512 || seq_k < 0) {
-        fail(-1, what, "need heads % kv_heads == 0, 0 < head_dim <= 512, seq_k >= 0");
+    if (kv_heads <= 0 || heads % kv_heads != 0 || head_dim <= 0 || head_dim > IRIS_ATTENTION_MAX_HEAD_DIM || seq_k < 0) {
+        fail(-1, what, "need heads % kv_heads == 0, 0 < head_dim <= 2048, seq_k >= 0");
         return;
     }
     if (wq && (!rope_cos || !rope_sin || (head_dim & 1))) {
@@ -231,40 +257,57 @@ static void attention(const char *what, uint16_t *out, int ldo,
             err = iris_hip_fa_hd128(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads,
                                     scale, causal != 0, key_mask);
         }
-    } else if (wq) {
-        /* a normalised copy of Q (rows of heads * head_dim) in private scratch, then the generic kernel,
-         * which takes a row stride of its own for q */
-        const int ldq = heads * head_dim;
-        const size_t need = (size_t)seq_q * ldq * sizeof(uint16_t);
-        if (need > g_q_scratch_bytes) {
-            if (g_q_scratch) {
-                check(hipStreamSynchronize(g_stream), "sync");
-                check(hipFree(g_q_scratch), "free");
-            }
-            g_q_scratch = NULL;
-            g_q_scratch_bytes = 0;
-            if (hipMalloc((void **)&g_q_scratch, need) != hipSuccess) {
-                (void)hipGetLastError();
-                g_q_scratch = NULL;
-                fail(-1, what, "scratch allocation failed");
-                return;
-            }
-            g_q_scratch_bytes = need;
-        }
+        if (err) check((hipError_t)err, "attention launch");
+        return;
+    }
+    /* Every other shape. Q normalised on the way in: a normalised copy of Q (rows of heads * head_dim) in
+     * private scratch takes the place of q from here on. */
+    const uint16_t *qq = q;
+    int ldq = ldi;
+    if (wq) {
+        ldq = heads * head_dim;
+        if (!scratch_fit((void **)&g_q_scratch, &g_q_scratch_bytes, (size_t)seq_q * ldq * sizeof(uint16_t), what)) return;
         if (!check(hipMemcpy2DAsync(g_q_scratch, (size_t)ldq * 2, q, (size_t)ldi * 2, (size_t)ldq * 2, (size_t)seq_q,
                                     hipMemcpyDeviceToDevice, g_stream), "copy of q"))
             return;
         norm_rope(g_q_scratch, NULL, ldq, wq, NULL, rope_cos, rope_sin, seq_q, heads, 0, head_dim, eps, split_half);
-        g_last_kernel = "attention_generic_qnorm";
-        err = iris_hip_attention_generic(g_stream, out, ldo, g_q_scratch, ldq, k, v, ldi, seq_q, seq_k, heads,
-                                         kv_heads, head_dim, scale, causal != 0, key_mask);
-    } else if (mfma_ok && (head_dim == 256 || head_dim == 512)) {
+        qq = g_q_scratch;
+    }
+    const int mfma_args = seq_k > 0 && scale > 0.0f && head_dim <= 512 && (!key_mask || seq_k <= IRIS_FA_MAX_MASKED_KEYS);
+    if (mfma_ok && !wq && (head_dim == 256 || head_dim == 512)) {
         g_last_kernel = "fa_sliced";
         err = iris_hip_fa_sliced(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads,
                                  head_dim, scale, causal != 0, key_mask);
+    } else if (mfma_args) {
+        /* Any head_dim <= 512, any stride and alignment: q | k | v copied into one fused row buffer with
+         * every head padded with zeros to the next of 128 / 256 / 512 dims, the matrix-core kernel of that
+         * width on the copy, and the first head_dim of every head's output columns copied back. */
+        const int hdp = head_dim <= 128 ? 128 : head_dim <= 256 ? 256 : 512;
+        const int rows = seq_q > seq_k ? seq_q : seq_k;
+        const int ldp = (heads + 2 * kv_heads) * hdp, ldop = heads * hdp;
+        const size_t in_bytes = ((size_t)rows * ldp * 2 + 255) & ~(size_t)255;
+        const int direct_out = head_dim == hdp && ldo % 4 == 0 && aligned(out, 8);
+        if (!scratch_fit((void **)&g_pack, &g_pack_bytes, in_bytes + (direct_out ? 0 : (size_t)seq_q * ldop * 2), what)) return;
+        uint16_t *packed = g_pack, *outp = direct_out ? out : g_pack + in_bytes / 2;
+        err = iris_hip_pack_heads(g_stream, packed, qq, ldq, seq_q, k, v, ldi, seq_k, heads, kv_heads, head_dim, hdp);
+        if (!err) {
+            const uint16_t *pk = packed + (size_t)heads * hdp, *pv = pk + (size_t)kv_heads * hdp;
+            const int ldout = direct_out ? ldo : ldop;
+            if (hdp == 128) {
+                g_last_kernel = wq ? "fa_hd128_packed_qnorm" : "fa_hd128_packed";
+                err = iris_hip_fa_hd128(g_stream, outp, ldout, packed, pk, pv, ldp, seq_q, seq_k, heads, kv_heads,
+                                        scale, causal != 0, key_mask);
+            } else {
+                g_last_kernel = wq ? "fa_sliced_packed_qnorm" : "fa_sliced_packed";
+                err = iris_hip_fa_sliced(g_stream, outp, ldout, packed, pk, pv, ldp, seq_q, seq_k, heads, kv_heads,
+                                         hdp, scale, causal != 0, key_mask);
+            }
+        }
+        if (!err && !direct_out)
+            err = iris_hip_unpack_heads(g_stream, out, ldo, outp, ldop, seq_q, heads, head_dim, hdp);
     } else {
-        g_last_kernel = "attention_generic";
-        err = iris_hip_attention_generic(g_stream, out, ldo, q, ldi, k, v, ldi, seq_q, seq_k, heads,
+        g_last_kernel = wq ? "attention_generic_qnorm" : "attention_generic";
+        err = iris_hip_attention_generic(g_stream, out, ldo, qq, ldq, k, v, ldi, seq_q, seq_k, heads,
                                          kv_heads, head_dim, scale, causal != 0, key_mask);
     }
     if (err) check((hipError_t)err, "attention launch");

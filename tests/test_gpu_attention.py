@@ -304,6 +304,25 @@ def test_vae_shape_full_size_sampled_rows(dev, orc):
     assert_close(O.bf16_to_f32(out2), np.tile(O.bf16_to_f32(buf[5, 2 * hd:]), (seq, 1)), "VAE shape constant V")
 
 
+def test_vae_shape_at_its_largest_50176_tokens(dev, orc):
+    """The largest image the reference decodes in one piece is 1792 x 1792: (1792 / 8)^2 = 50176 tokens through the
+    mid-block attention (iris_vae.c:1112-1124), one head of 512. Sampled rows against the oracle (first and last
+    workgroups, workgroup boundaries) and constant V over all rows."""
+    seq, hd = 50176, 512
+    buf, ldi = random_case(78, seq, seq, 1, 1, hd=hd)
+    scale = float(1 / np.sqrt(hd))
+    out, kernel = dev.attention(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale)
+    assert kernel == "fa_sliced"
+    rows = np.unique(np.r_[sample_rows(seq, n=10), [63, 64, 25087, 25088, seq - 65, seq - 64]]).astype(np.int32)
+    want = orc.attention_bf16(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale, rows=rows)
+    assert_close(O.bf16_to_f32(out[rows]), want, "VAE 50176 tokens sampled")
+    buf[:, 2 * hd:] = buf[5, 2 * hd:]
+    out2, _ = dev.attention(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale)
+    got2 = O.bf16_to_f32(out2)
+    assert np.array_equal(got2, np.tile(got2[0], (seq, 1)))
+    assert_close(got2[:4], np.tile(O.bf16_to_f32(buf[5, 2 * hd:]), (4, 1)), "VAE 50176 tokens constant V")
+
+
 def test_sliced_kernel_empty_rows_and_large_scores(dev, orc):
     seq, hd = 100, 512
     buf, ldi = random_case(21, seq, seq, 1, 1, hd=hd, sigma=3.0)          # |score| up to ~100
@@ -319,8 +338,13 @@ def test_sliced_kernel_empty_rows_and_large_scores(dev, orc):
 
 
 @pytest.mark.parametrize("hd,heads,kv,causal,masked", [(64, 4, 4, False, False), (64, 4, 2, True, True),
-                                                       (384, 1, 1, False, False), (96, 2, 1, True, False)])
-def test_generic_kernel_other_head_dims(dev, orc, hd, heads, kv, causal, masked):
+                                                       (384, 1, 1, False, False), (96, 2, 1, True, False),
+                                                       (40, 3, 3, False, True), (2, 2, 1, False, False),
+                                                       (130, 2, 2, True, True), (200, 4, 2, False, False)])
+def test_other_head_dims_run_on_the_matrix_cores_through_a_padded_copy(dev, orc, hd, heads, kv, causal, masked):
+    """Head sizes other than 128 / 256 / 512 (odd ones included): q, k and v are copied into a fused row
+    buffer with every head padded with zeros to the next of those sizes, the matrix-core kernel of that
+    size runs on the copy, and the first head_dim output columns of every head are copied back."""
     seq = 150
     buf, ldi = random_case(hd + heads, seq, seq, heads, kv, hd=hd)
     qd, kd = heads * hd, kv * hd
@@ -328,19 +352,64 @@ def test_generic_kernel_other_head_dims(dev, orc, hd, heads, kv, causal, masked)
     if masked:
         mask = (np.arange(seq) < 101).astype(np.int32)
     scale = 1 / np.sqrt(hd)
+    ldo = heads * hd + 3
+    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq, seq, heads, kv, hd, scale, causal, mask, ldo=ldo)
+    assert kernel == ("fa_hd128_packed" if hd <= 128 else "fa_sliced_packed")
+    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq, seq, heads, kv, hd, scale, causal, mask)
+    assert_close(O.bf16_to_f32(out[:, :heads * hd]), want, f"padded copy hd={hd}")
+    assert np.all(out[:, heads * hd:] == 0x7fc0)              # nothing written past the head columns
+
+
+@pytest.mark.parametrize("hd,pad,qoff", [(128, 3, 0), (128, 0, 1), (512, 5, 0), (256, 8, 3)])
+def test_misaligned_rows_run_on_the_matrix_cores_through_an_aligned_copy(dev, orc, hd, pad, qoff):
+    """A row stride that is not a multiple of 8 elements, or q / k / v that do not start on 16 bytes."""
+    heads, seq = 2, 70
+    buf, ldi = random_case(13 + hd + pad, seq, seq, heads, heads, hd=hd, pad=pad + qoff)
+    qd = heads * hd
+    scale = float(1 / np.sqrt(hd))
+    out, kernel = dev.attention(buf, ldi, qoff, qoff + qd, qoff + 2 * qd, seq, seq, heads, heads, hd, scale)
+    assert kernel == ("fa_hd128_packed" if hd == 128 else "fa_sliced_packed")
+    want = orc.attention_bf16(buf, ldi, qoff, qoff + qd, qoff + 2 * qd, seq, seq, heads, heads, hd, scale)
+    assert_close(O.bf16_to_f32(out), want, f"misaligned hd={hd} pad={pad} offset={qoff}")
+
+
+def test_padded_copy_with_fewer_queries_than_keys_and_large_sizes(dev, orc):
+    """seq_q != seq_k (the fused copy has max(seq_q, seq_k) rows) and a size where the copy is grown."""
+    for seq_q, seq_k, hd, heads, kv in ((45, 333, 64, 4, 2), (700, 90, 96, 2, 2), (2000, 2000, 64, 8, 8)):
+        buf, ldi = random_case(seq_q + seq_k, seq_q, seq_k, heads, kv, hd=hd)
+        qd, kd = heads * hd, kv * hd
+        scale = float(1 / np.sqrt(hd))
+        out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale)
+        assert kernel == "fa_hd128_packed"
+        rows = sample_rows(seq_q, n=12) if seq_q > 300 else np.arange(seq_q, dtype=np.int32)
+        rows = rows[(rows >= 0) & (rows < seq_q)]
+        want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, rows=rows)
+        assert_close(O.bf16_to_f32(out[:seq_q])[rows], want, f"padded copy {seq_q}x{seq_k}")
+
+
+@pytest.mark.parametrize("hd,heads,kv,causal", [(640, 2, 1, True), (1024, 1, 1, False), (2048, 1, 1, False), (1100, 2, 2, False)])
+def test_head_dims_beyond_512_on_the_scalar_kernel(dev, orc, hd, heads, kv, causal):
+    """The reference answers any head_dim (its fallback is two GEMMs); here sizes beyond the matrix-core kernels'
+    512 go to the scalar kernel, which walks the dims in chunks of 512, up to 2048."""
+    seq = 70
+    buf, ldi = random_case(hd, seq, seq, heads, kv, hd=hd)
+    qd, kd = heads * hd, kv * hd
+    scale = float(1 / np.sqrt(hd))
+    mask = (np.arange(seq) != 7).astype(np.int32)
     out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq, seq, heads, kv, hd, scale, causal, mask)
     assert kernel == "attention_generic"
     want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq, seq, heads, kv, hd, scale, causal, mask)
-    assert_close(O.bf16_to_f32(out), want, f"generic hd={hd}")
+    assert_close(O.bf16_to_f32(out), want, f"scalar hd={hd}")
 
 
-def test_misaligned_stride_falls_back_not_fails(dev, orc):
+def test_scalar_kernel_still_answers_what_the_matrix_cores_cannot(dev, orc):
+    """A non-positive scale (the matrix-core kernels fold the scale into the exponent base) goes to the scalar kernel."""
     heads, seq = 2, 40
-    buf, ldi = random_case(13, seq, seq, heads, heads, pad=3)      # ldi % 8 != 0
-    out, kernel = dev.attention(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, 0.0884)
+    buf, ldi = random_case(13, seq, seq, heads, heads)
+    out, kernel = dev.attention(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, -0.0884)
     assert kernel == "attention_generic"
-    want = orc.attention_bf16(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, 0.0884)
-    assert_close(O.bf16_to_f32(out), want, "misaligned")
+    want = orc.attention_bf16(buf, ldi, 0, 256, 512, seq, seq, heads, heads, 128, -0.0884)
+    assert_close(O.bf16_to_f32(out), want, "negative scale")
 
 
 def test_bad_arguments_are_reported_not_fatal(dev):
@@ -348,5 +417,7 @@ def test_bad_arguments_are_reported_not_fatal(dev):
     d = dev.put(buf)
     dev.lib.iris_dev_last_error()
     dev.lib.iris_dev_attention(d, 384, d, d, d, ldi, 8, 8, 3, 2, 128, 0.1, 0, None)    # 3 % 2 != 0
+    assert dev.lib.iris_dev_last_error() != 0
+    dev.lib.iris_dev_attention(d, 4096, d, d, d, ldi, 8, 8, 1, 1, 2049, 0.1, 0, None)   # head_dim beyond the limit
     assert dev.lib.iris_dev_last_error() != 0
     dev.free_all()

@@ -111,8 +111,8 @@ def test_fewer_queries_than_keys(dev):
 
 @pytest.mark.parametrize("hd,ldi_extra,split", [(64, 0, 0), (64, 0, 1), (128, 2, 0), (256, 0, 1)])
 def test_other_shapes_go_through_the_normalised_copy(dev, orc, hd, ldi_extra, split):
-    """head_dim != 128 or rows that are not 16-byte aligned: a normalised copy of Q in private scratch and the generic
-    kernel; checked against the oracle, q untouched."""
+    """head_dim != 128 or rows that are not 16-byte aligned: a normalised copy of Q in private scratch, then the
+    padded copy and the matrix-core kernel; checked against the oracle, q untouched."""
     rng = np.random.default_rng(hd + ldi_extra)
     seq, heads, kv = 70, 4, 2
     q_dim, kv_dim = heads * hd, kv * hd
@@ -124,7 +124,7 @@ def test_other_shapes_go_through_the_normalised_copy(dev, orc, hd, ldi_extra, sp
     mask = (rng.random(seq) < 0.8).astype(np.int32); mask[0] = 1
     got, kernel, after = dev.attention_qnorm(buf, ldi, 0, q_dim, q_dim + kv_dim, seq, seq, heads, kv, hd, scale, w,
                                              np.cos(ang), np.sin(ang), 1e-5, split, causal=True, key_mask=mask)
-    assert kernel == "attention_generic_qnorm"
+    assert kernel == ("fa_hd128_packed_qnorm" if hd <= 128 else "fa_sliced_packed_qnorm")
     assert np.array_equal(after, buf)
     ref = buf.copy()
     orc.head_norm_rope_bf16(ref, ldi, w, np.cos(ang), np.sin(ang), seq, heads, hd, 1e-5, split, col0=0)
@@ -143,7 +143,7 @@ def test_scratch_copy_grows_and_is_reused(dev, orc):
         w = np.ones(hd, np.float32)
         got, kernel, _ = dev.attention_qnorm(buf, ldi, 0, heads * hd, 2 * heads * hd, seq, seq, heads, heads, hd, 0.125, w,
                                              np.cos(ang), np.sin(ang), 1e-6, 0)
-        assert kernel == "attention_generic_qnorm"
+        assert kernel == "fa_hd128_packed_qnorm"
         ref = buf.copy()
         orc.head_norm_rope_bf16(ref, ldi, w, np.cos(ang), np.sin(ang), seq, heads, hd, 1e-6, 0, col0=0)
         want = orc.attention_bf16(ref, ldi, 0, heads * hd, 2 * heads * hd, seq, seq, heads, heads, hd, 0.125)
