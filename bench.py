@@ -270,9 +270,30 @@ def other_ops(dev, hip, stream, rng, settle_ms=0.0):
                 ms = timed(lambda i: fn(y, x, W, rows, k, n), 5)
                 res.append({"op": name, "kernel": dev.last_kernel(), "shape": f"{rows}x{k}->{n}", "us": round(ms * 1e3, 1),
                             "tflops": round(2 * rows * k * n / ms / 1e9, 1)})
-    lib.iris_dev_linear_backend(0)
-    xf, af = _vp(y), _vp(y + rows * dim * 4)
+    # the fused q | k | v (| gate | up) projection with the norm+rope of its Q and K columns: the reference's three calls
+    # (iris_transformer_flux.c:3833-3837) and the entry that takes them as one
     w1 = dev.to_device(np.ones(dim, np.float32))
+    ang = rng.uniform(-3.0, 3.0, (rows, 64)).astype(np.float32)
+    cos, sin = dev.to_device(np.cos(ang)), dev.to_device(np.sin(ang))
+    heads = dim // 128
+    for n in (9216, 27648):
+        def three_calls(i):
+            lib.iris_dev_linear_bf16(y, x, W, rows, dim, n)
+            lib.iris_dev_head_norm_rope(y, n, w1, cos, sin, rows, heads, 128, 1e-6, 0)
+            lib.iris_dev_head_norm_rope(_vp(y + 2 * dim), n, w1, cos, sin, rows, heads, 128, 1e-6, 0)
+
+        def one_call(i):
+            lib.iris_dev_linear_bf16_qknorm(y, x, W, rows, dim, n, heads, heads, 128, w1, w1, cos, sin, 1e-6, 0)
+        for backend in (0, 1):
+            lib.iris_dev_linear_backend(backend)
+            for name, fn in (("linear_bf16 + 2 x head_norm_rope", three_calls), ("linear_bf16_qknorm", one_call)):
+                ms = timed(fn, 5)
+                res.append({"op": name, "linear_backend": backend, "kernel": dev.last_kernel(), "shape": f"{rows}x{dim}->{n}",
+                            "us": round(ms * 1e3, 1)})
+    lib.iris_dev_linear_backend(0)
+    for p in (cos, sin):
+        lib.iris_dev_free(p)
+    xf, af = _vp(y), _vp(y + rows * dim * 4)
     ob = _vp(x)
     n = rows * dim
     one_pass = [("layer_norm_mod", lambda i: lib.iris_dev_layer_norm_mod(ob, xf, w1, w1, rows, dim, 1e-6), 6 * n),

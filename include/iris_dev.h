@@ -171,6 +171,25 @@ void iris_dev_attention_qnorm(uint16_t *out, int ldo,
                               const float *wq, const float *rope_cos, const float *rope_sin,
                               float eps, int split_half);
 
+/* The projection and the normalisation of its output as one launch: the result is what
+ *     iris_dev_linear_bf16(y, x, W, rows, in, out);
+ *     iris_dev_head_norm_rope_qk(y, y + q_heads * head_dim, out, wq, wk, rope_cos, rope_sin,
+ *                                rows, q_heads, k_heads, head_dim, eps, split_half);
+ * gives: the leading q_heads * head_dim columns of y are Q heads, the next k_heads * head_dim columns K heads,
+ * the rest (V, and the MLP columns of the fused single-block projection) is stored as the projection leaves
+ * it. This is the layout of every fused QKV projection of the reference's device paths
+ * (iris_transformer_flux.c:3795-3800 and 3833-3837, iris_transformer_flux3.c:692-694,
+ * iris_transformer_zimage.c:1947-1949, iris_qwen3.c:1589-1593), which all issue exactly these three calls. The
+ * library's own GEMM can normalise each 256 x 256 output tile while it still sits in the LDS, which saves the
+ * pass that reads and rewrites the Q and K rows: that one-launch kernel runs when the own GEMM is selected
+ * (iris_dev_linear_backend(1)) or the vendor library is absent, for head_dim 128, rows >= 256, out >= 256 and
+ * a multiple of 128, in a multiple of 64 and 16-byte aligned operands; its bits are those of the two calls
+ * above on the own GEMM. Otherwise the entry issues the two calls itself (the vendor GEMM followed by the norm
+ * kernel is the faster pair where that library is present). */
+void iris_dev_linear_bf16_qknorm(uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out,
+                                 int q_heads, int k_heads, int head_dim, const float *wq, const float *wk,
+                                 const float *rope_cos, const float *rope_sin, float eps, int split_half);
+
 /* The library's stream as a hipStream_t, for callers that time kernels with
  * HIP events or order their own work after the library's. */
 void *iris_dev_stream(void);

@@ -34,6 +34,7 @@ ABI = {
     "iris_dev_f32_to_bf16": (None, [_vp, _vp, _sz]),
     "iris_dev_linear_f32": (None, [_vp, _vp, _vp, _i, _i, _i]),
     "iris_dev_linear_bf16": (None, [_vp, _vp, _vp, _i, _i, _i]),
+    "iris_dev_linear_bf16_qknorm": (None, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _f, _i]),
     "iris_dev_layer_norm_mod": (None, [_vp, _vp, _vp, _vp, _i, _i, _f]),
     "iris_dev_rms_norm": (None, [_vp, _vp, _vp, _i, _i, _f]),
     "iris_dev_rms_norm_mod": (None, [_vp, _vp, _vp, _vp, _i, _i, _f]),

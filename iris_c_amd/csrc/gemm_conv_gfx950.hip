@@ -35,6 +35,7 @@
 #include <stdint.h>
 
 #include "iris_kernels_hip.h"
+#include "norm_rope_math.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -189,14 +190,24 @@ __device__ __forceinline__ uint32_t lds_address(const uint16_t *p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
 }
 
+/* The per-head RMSNorm + rotary embedding of the leading columns of a projection, applied by the GEMM to its
+ * own output tile (head_dim 128): columns [0, q_cols) are heads normalised with wq, [q_cols, qk_cols) with wk,
+ * the rest is stored as it is. */
+struct QkNorm {
+    const float *wq, *wk, *rope_cos, *rope_sin;  /* [128], [128], [M, 64], [M, 64] */
+    int q_cols, qk_cols;
+    float eps;
+    int split_half;
+};
+
 /* M0 (the LDS address of a direct load) is named as clobbered by the asm statements below; the
  * compiler reserves that register for its own short-lived uses and remarks on it. */
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-template <typename OUT, int TN, bool CONV>
+template <typename OUT, int TN, bool CONV, bool QKN = false>
 __global__ void __launch_bounds__(512, 2)
 k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *__restrict__ W,
-           int M, int N, int K, int tiles_m, int total, int per_xcd, ConvGeom geo) {
+           int M, int N, int K, int tiles_m, int total, int per_xcd, ConvGeom geo, QkNorm qn) {
     constexpr int WAVES_N = TN / 64, WAVES_M = 8 / WAVES_N;    /* wave grid */
     constexpr int NB = DT / WAVES_M / 16;                      /* x blocks (16 rows) per wave: 8 or 4 */
     constexpr int HALVES = NB / 4;
@@ -362,6 +373,60 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
      * LDS serves a wave's instructions in order, so the reads see the writes without a barrier. */
     constexpr int PER16 = 16 / (int)sizeof(OUT);               /* outputs per 16 B */
     const int mw = m0 + 16 * NB * wm, nw = n0 + 64 * wn;
+    if constexpr (QKN) {
+        /* A head (128 columns) spans the blocks of two waves, so a tile with head columns in it is staged as a
+         * whole: 256 rows x 512 B fill the 128 KB exactly. 16 B chunk c of row r sits in slot
+         * (c & 16) | ((c ^ r) & 15): the 16 rows of a write and the 16 chunks of a head vector both spread over
+         * all banks. Then a 16-lane row per (token, head) vector, 32 vectors a pass, through the same function
+         * as the stand-alone kernel: the stored bits are those of the plain projection followed by that kernel. */
+        static_assert(sizeof(OUT) == 2 && TN == 256 && !CONV, "bf16 projection tiles of 256 x 256 only");
+        if (n0 < qn.qk_cols) {                                  /* the same for the whole workgroup */
+#pragma unroll
+            for (int b = 0; b < NB; b++)
+#pragma unroll
+                for (int a = 0; a < 4; a++) {
+                    const int row = 16 * NB * wm + 16 * b + li, chunk = 8 * wn + 2 * a + (lg >> 1);
+                    const int slot = (chunk & 16) | ((chunk ^ li) & 15);
+                    *reinterpret_cast<uint2 *>(&dlds[row * 256 + 8 * slot + 4 * (lg & 1)]) =
+                        make_uint2(pack_bf16(acc[a][b][0], acc[a][b][1]), pack_bf16(acc[a][b][2], acc[a][b][3]));
+                }
+            __syncthreads();
+            const int sub = tid & 15, head = (tid >> 4) & 1, row_in = tid >> 5;
+            const int n_head = n0 + 128 * head, n = n_head + 8 * sub;
+            const bool normed = n_head < qn.qk_cols;
+            float w8[8] = {};
+            if (normed) {
+                const float *wsel = (n_head < qn.q_cols ? qn.wq : qn.wk) + 8 * sub;
+                const float4 w0 = *reinterpret_cast<const float4 *>(wsel), w1 = *reinterpret_cast<const float4 *>(wsel + 4);
+                w8[0] = w0.x; w8[1] = w0.y; w8[2] = w0.z; w8[3] = w0.w; w8[4] = w1.x; w8[5] = w1.y; w8[6] = w1.z; w8[7] = w1.w;
+            }
+            const int tcol = qn.split_half ? 8 * (sub & 7) : 4 * sub;
+            const int chunk = 16 * head + sub;
+#pragma unroll 4
+            for (int pass = 0; pass < DT / 16; pass++) {
+                const int row = 16 * pass + row_in, m = m0 + row;
+                if (m >= M || n_head >= N) continue;            /* the same for the 16 lanes of a vector */
+                u32x4 v = *reinterpret_cast<const u32x4 *>(&dlds[row * 256 + 8 * ((chunk & 16) | ((chunk ^ row) & 15))]);
+                if (normed) {
+                    const float *cr = qn.rope_cos + (size_t)m * 64 + tcol, *sr = qn.rope_sin + (size_t)m * 64 + tcol;
+                    float cv[8] = {}, sv[8] = {};
+                    const float4 c0 = *reinterpret_cast<const float4 *>(cr), s0 = *reinterpret_cast<const float4 *>(sr);
+                    cv[0] = c0.x; cv[1] = c0.y; cv[2] = c0.z; cv[3] = c0.w;
+                    sv[0] = s0.x; sv[1] = s0.y; sv[2] = s0.z; sv[3] = s0.w;
+                    if (qn.split_half) {
+                        const float4 c1 = *reinterpret_cast<const float4 *>(cr + 4), s1 = *reinterpret_cast<const float4 *>(sr + 4);
+                        cv[4] = c1.x; cv[5] = c1.y; cv[6] = c1.z; cv[7] = c1.w;
+                        sv[4] = s1.x; sv[5] = s1.y; sv[6] = s1.z; sv[7] = s1.w;
+                        v = nr_vector_hd128<true>(v, w8, cv, sv, qn.eps, sub);
+                    } else {
+                        v = nr_vector_hd128<false>(v, w8, cv, sv, qn.eps, sub);
+                    }
+                }
+                *reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(y) + (size_t)m * N + n) = v;
+            }
+            return;
+        }
+    }
     const float *bias = CONV ? geo.bias : nullptr;
     const bool staged = N % PER16 == 0 && ((uintptr_t)y & 15) == 0;
     if (staged) {
@@ -425,19 +490,20 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
 
 constexpr int DMA_LDS_BYTES = 128 * 1024;        /* two stages of (256 + 256) x 128 B; also the 8 x 16 KB of the epilogue */
 
-template <typename OUT, int TN, bool CONV>
-int launch_gemm_dma(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, int N, int K, const ConvGeom &geo) {
+template <typename OUT, int TN, bool CONV, bool QKN = false>
+int launch_gemm_dma(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, int N, int K, const ConvGeom &geo,
+                    const QkNorm &qn = QkNorm{}) {
     static bool configured = false;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_dma<OUT, TN, CONV>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_dma<OUT, TN, CONV, QKN>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, DMA_LDS_BYTES);
         if (e != hipSuccess) return (int)e;
         configured = true;
     }
     const int tiles_m = (M + DT - 1) / DT, tiles_n = (N + TN - 1) / TN, total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) / 8;
-    hipLaunchKernelGGL((k_gemm_dma<OUT, TN, CONV>), dim3((unsigned)per_xcd * 8), dim3(512), DMA_LDS_BYTES, st, y, x, W, M, N, K,
-                       tiles_m, total, per_xcd, geo);
+    hipLaunchKernelGGL((k_gemm_dma<OUT, TN, CONV, QKN>), dim3((unsigned)per_xcd * 8), dim3(512), DMA_LDS_BYTES, st, y, x, W, M, N, K,
+                       tiles_m, total, per_xcd, geo, qn);
     return (int)hipGetLastError();
 }
 
@@ -524,6 +590,24 @@ int iris_hip_linear_bf16(void *stream, uint16_t *y, const uint16_t *x, const uin
 
 /* Zeroes the first IRIS_CONV_ZERO_BYTES of a freshly allocated convolution scratch buffer: the page that taps
  * outside the image read. iris_hip_conv2d never writes there. */
+/* y = x W^T as bf16 with the per-head RMSNorm + rotary embedding (head_dim 128) of columns [0, q_cols) (weights
+ * wq) and [q_cols, q_cols + k_cols) (weights wk) applied in the GEMM's epilogue. Returns -2, with nothing
+ * enqueued, for a shape the tiled kernel does not take: the caller then runs the two steps one after the other. */
+int iris_hip_linear_bf16_qknorm(void *stream, uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out,
+                                int q_cols, int k_cols, const float *wq, const float *wk, const float *rope_cos,
+                                const float *rope_sin, float eps, int split_half) {
+    const int M = rows, N = out, K = in;
+    const uintptr_t all = (uintptr_t)x | (uintptr_t)W | (uintptr_t)y | (uintptr_t)wq | (uintptr_t)wk | (uintptr_t)rope_cos |
+                          (uintptr_t)rope_sin;
+    const bool tiled = K > 0 && K % TK == 0 && (all & 15) == 0 && M >= DT && N >= DT && (size_t)K * 2 * 8 < ((size_t)1 << 31);
+    if (!tiled || N % 128 || q_cols < 0 || k_cols < 0 || q_cols % 128 || k_cols % 128 || q_cols + k_cols > N ||
+        q_cols + k_cols == 0)
+        return -2;
+    const ConvGeom none = {};
+    const QkNorm qn = {wq, k_cols ? wk : wq, rope_cos, rope_sin, q_cols, q_cols + k_cols, eps, split_half};
+    return launch_gemm_dma<uint16_t, 256, false, true>((hipStream_t)stream, y, x, W, M, N, K, none, qn);
+}
+
 int iris_hip_conv2d_prepare_scratch(void *stream, uint16_t *scratch) {
     hipLaunchKernelGGL(k_zero_words, dim3(1), dim3(64), 0, (hipStream_t)stream, reinterpret_cast<uint32_t *>(scratch),
                        IRIS_CONV_ZERO_BYTES / 4);

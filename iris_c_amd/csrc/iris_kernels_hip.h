@@ -111,6 +111,10 @@ int iris_hip_group_norm_static(void *stream, float *out, const float *in, const 
  * x, W are 16-byte aligned, scalar kernel otherwise */
 int iris_hip_linear_f32(void *stream, float *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out);
 int iris_hip_linear_bf16(void *stream, uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out);
+/* -2 = shape not taken, nothing enqueued */
+int iris_hip_linear_bf16_qknorm(void *stream, uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out,
+                                int q_cols, int k_cols, const float *wq, const float *wk, const float *rope_cos,
+                                const float *rope_sin, float eps, int split_half);
 /* Convolution. `scratch` is a private device buffer, 16-byte aligned, whose first IRIS_CONV_ZERO_BYTES are zeroed
  * once by iris_hip_conv2d_prepare_scratch and never written again (the page that taps outside the image read);
  * the rest holds the image as bf16 (or the bf16 patches of the shapes that are gathered: >= 2 * k * k * cin bytes). */

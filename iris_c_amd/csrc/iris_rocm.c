@@ -377,6 +377,36 @@ void iris_dev_linear_bf16(uint16_t *y, const uint16_t *x, const uint16_t *W, int
     LAUNCH("linear", iris_hip_linear_bf16(g_stream, y, x, W, rows, in, out));
 }
 
+void iris_dev_linear_bf16_qknorm(uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out,
+                                 int q_heads, int k_heads, int head_dim, const float *wq, const float *wk,
+                                 const float *rope_cos, const float *rope_sin, float eps, int split_half) {
+    if (rows <= 0 || out <= 0) return;
+    if (in <= 0) { fail(-1, "linear_qknorm", "in must be positive"); return; }
+    if (q_heads < 0 || k_heads < 0 || head_dim <= 0 || (long long)(q_heads + k_heads) * head_dim > out) {
+        fail(-1, "linear_qknorm", "need (q_heads + k_heads) * head_dim <= out");
+        return;
+    }
+    if (!need_ready("linear_qknorm")) return;
+    /* With the vendor GEMM selected and present, its linear layer followed by the norm kernel is the faster pair
+     * (4608 rows, 3072 -> 9216: 215 us against 225 us for the one-launch kernel, whose GEMM is the library's
+     * own: 199 + 17 against 220 + 7); with the own GEMM selected the one launch saves 11 us of 238. */
+    int one_launch = head_dim == 128 && q_heads + k_heads > 0 &&
+                     (g_linear_backend != 0 || !iris_lt_available() || in % 8 != 0);
+    if (one_launch) {
+        int err = iris_hip_linear_bf16_qknorm(g_stream, y, x, W, rows, in, out, q_heads * 128, k_heads * 128, wq, wk,
+                                              rope_cos, rope_sin, eps, split_half != 0);
+        if (err == 0) { g_last_kernel = "linear_mfma_qknorm"; return; }
+        if (err != -2) { check((hipError_t)err, "linear_qknorm launch"); return; }
+    }
+    /* the two steps one after the other */
+    iris_dev_linear_bf16(y, x, W, rows, in, out);
+    if (q_heads > 0)
+        norm_rope(y, k_heads ? y + (size_t)q_heads * head_dim : NULL, out, wq, wk, rope_cos, rope_sin, rows, q_heads, k_heads,
+                  head_dim, eps, split_half);
+    else if (k_heads > 0)
+        norm_rope(y, NULL, out, wk, NULL, rope_cos, rope_sin, rows, k_heads, 0, head_dim, eps, split_half);
+}
+
 void iris_dev_layer_norm_mod(uint16_t *out, const float *x, const float *shift, const float *scale,
                              int rows, int dim, float eps) {
     LAUNCH("layer_norm_mod", iris_hip_layer_norm_mod(g_stream, out, x, shift, scale, rows, dim, eps));

@@ -24,8 +24,6 @@
 #include "iris_kernels_hip.h"
 #include "norm_rope_math.h"
 
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
@@ -36,30 +34,6 @@ constexpr int kThreads = 256;
  * the units) is within 3 % either way; nontemporal loads cost 5 %. */
 constexpr int kUnroll = 2;                       /* vectors in flight per 16-lane row */
 constexpr int kUnitsPerBlock = (kThreads / 16) * kUnroll;
-
-__device__ __forceinline__ float bf_lo(uint32_t u) { return __uint_as_float(u << 16); }
-__device__ __forceinline__ float bf_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
-
-/* Two f32 -> packed bf16x2, round to nearest even (v_cvt_pk_bf16_f32; equals
- * the integer form u += 0x7fff + ((u >> 16) & 1) for every finite input). */
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    f32x2 p = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2));
-}
-
-/* Sum over the 16 lanes of a DPP row; every lane gets the total. */
-__device__ __forceinline__ float row16_sum(float v) {
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));
-    return v;
-}
-
-/* The value held by the lane 8 places away in the same 16-lane row. */
-__device__ __forceinline__ float row16_partner8(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
-}
 
 template <bool SPLIT>
 __global__ void __launch_bounds__(kThreads)
@@ -74,7 +48,6 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
     /* Table columns this lane needs: consecutive pairs -> i = 4*sub..4*sub+3;
      * split-half -> i = 8*(sub&7)..+7 (shared with the partner lane). */
     const int tcol = SPLIT ? 8 * (sub & 7) : 4 * sub;
-    const float sgn = (SPLIT && sub < 8) ? -1.0f : 1.0f;
 
     /* Phase 1: request everything this thread needs for its kUnroll vectors --
      * the 16 B of x and the matching cos/sin entries -- before touching any of
@@ -120,40 +93,15 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
         if (!ptr[u]) continue;
-        float e[8] = {bf_lo(raw[u].x), bf_hi(raw[u].x), bf_lo(raw[u].y), bf_hi(raw[u].y),
-                      bf_lo(raw[u].z), bf_hi(raw[u].z), bf_lo(raw[u].w), bf_hi(raw[u].w)};
-        const float ss = row16_sum(nr_chunk_sum_squares(e));
-        const float inv = nr_inv_rms128(ss, eps);
+        float cv[8], sv[8];
+        cv[0] = ct[u][0].x; cv[1] = ct[u][0].y; cv[2] = ct[u][0].z; cv[3] = ct[u][0].w;
+        cv[4] = ct[u][TN - 1].x; cv[5] = ct[u][TN - 1].y; cv[6] = ct[u][TN - 1].z; cv[7] = ct[u][TN - 1].w;
+        sv[0] = st[u][0].x; sv[1] = st[u][0].y; sv[2] = st[u][0].z; sv[3] = st[u][0].w;
+        sv[4] = st[u][TN - 1].x; sv[5] = st[u][TN - 1].y; sv[6] = st[u][TN - 1].z; sv[7] = st[u][TN - 1].w;
+        float w8[8];
 #pragma unroll
-        for (int i = 0; i < 8; i++) e[i] = nr_scaled(e[i], inv, isk[u] ? wk8[i] : wq8[i]);
-
-        float o[8];
-        if (SPLIT) {
-            const float cv[8] = {ct[u][0].x, ct[u][0].y, ct[u][0].z, ct[u][0].w, ct[u][TN - 1].x, ct[u][TN - 1].y, ct[u][TN - 1].z, ct[u][TN - 1].w};
-            const float sv[8] = {st[u][0].x, st[u][0].y, st[u][0].z, st[u][0].w, st[u][TN - 1].x, st[u][TN - 1].y, st[u][TN - 1].z, st[u][TN - 1].w};
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                /* lanes 0-7 hold a (first half), lanes 8-15 hold b: a*c - b*s / b*c + a*s */
-                /* nr_rot_first(e, other) on the a lanes, nr_rot_second(other, e) on the b lanes, as one
-                 * expression: the sign flip is exact */
-                const float other = row16_partner8(e[i]);
-                o[i] = fmaf(sgn * other, sv[i], e[i] * cv[i]);
-            }
-        } else {
-            const float cv[4] = {ct[u][0].x, ct[u][0].y, ct[u][0].z, ct[u][0].w};
-            const float sv[4] = {st[u][0].x, st[u][0].y, st[u][0].z, st[u][0].w};
-#pragma unroll
-            for (int p = 0; p < 4; p++) {
-                const float a = e[2 * p], b = e[2 * p + 1];
-                o[2 * p] = nr_rot_first(a, b, cv[p], sv[p]);
-                o[2 * p + 1] = nr_rot_second(a, b, cv[p], sv[p]);
-            }
-        }
-        u32x4 out;
-        out.x = pack_bf16(o[0], o[1]);
-        out.y = pack_bf16(o[2], o[3]);
-        out.z = pack_bf16(o[4], o[5]);
-        out.w = pack_bf16(o[6], o[7]);
+        for (int i = 0; i < 8; i++) w8[i] = isk[u] ? wk8[i] : wq8[i];
+        const u32x4 out = nr_vector_hd128<SPLIT>(raw[u], w8, cv, sv, eps, sub);
         /* Write-through store (sc0 sc1): the rows leave the L2 as they are produced instead of at the
          * end-of-kernel write-back, 2-5 % faster on 59-118 MB calls whether the rows were cached or not.
          * (Adding the streaming hint `nt` takes the two-tensor call on uncached rows from 23.0 to 21.2 us
@@ -181,7 +129,7 @@ k_norm_rope_generic(uint16_t *x, int ld, const float *w, const float *rope_cos,
         float a = __uint_as_float((uint32_t)v[i0] << 16) * (inv * w[i0]);
         float b = __uint_as_float((uint32_t)v[i1] << 16) * (inv * w[i1]);
         float c = rope_cos[(size_t)s * half + i], sn = rope_sin[(size_t)s * half + i];
-        uint32_t packed = pack_bf16(fmaf(-b, sn, a * c), fmaf(a, sn, b * c));
+        uint32_t packed = nr_pack_bf16(fmaf(-b, sn, a * c), fmaf(a, sn, b * c));
         v[i0] = (uint16_t)(packed & 0xffffu);
         v[i1] = (uint16_t)(packed >> 16);
     }

@@ -60,6 +60,7 @@ def test_no_gpu_means_no_silent_fallback(lib):
     lib.iris_dev_attention_qnorm(None, 0, None, None, None, 0, 4, 4, 1, 1, 128, 1.0, 0, None, None, None, None, 1e-6, 0)
     assert lib.iris_dev_last_error() != 0
     lib.iris_dev_linear_bf16(None, None, None, 4, 8, 4)
+    lib.iris_dev_linear_bf16_qknorm(None, None, None, 4, 8, 4, 1, 1, 2, None, None, None, None, 1e-6, 0)
     assert lib.iris_dev_last_error() != 0
     lib.iris_dev_conv2d(None, None, None, None, 4, 4, 64, 128, 3, 1, 1, 1)
     assert lib.iris_dev_last_error() != 0

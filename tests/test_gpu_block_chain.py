@@ -54,7 +54,7 @@ def oracle_block(orc, b):
     return orc.dev_residual(b["x"], out, b["mod"][2 * dim:])
 
 
-def device_block(dev, b, q_norm_inside_attention):
+def device_block(dev, b, q_norm_inside_attention, norm_inside_projection=False):
     lib = dev.lib
     seq, dim, mlp, ldh, ldc, heads = b["seq"], b["dim"], b["mlp"], b["ldh"], b["ldc"], b["heads"]
     x, mod = dev.put(b["x"]), dev.put(b["mod"])
@@ -63,16 +63,21 @@ def device_block(dev, b, q_norm_inside_attention):
     norm, h, cat, out = dev.alloc(seq * dim * 2), dev.alloc(seq * ldh * 2), dev.alloc(seq * ldc * 2), dev.alloc(seq * dim * 4)
     col = lambda p, elems: ptr_add(p, 2 * elems)
     lib.iris_dev_layer_norm_mod(norm, x, mod, ptr_add(mod, 4 * dim), seq, dim, 1e-6)
-    lib.iris_dev_linear_bf16(h, norm, w_in, seq, dim, ldh)
-    if q_norm_inside_attention:
+    projection = None
+    if norm_inside_projection:
+        lib.iris_dev_linear_bf16_qknorm(h, norm, w_in, seq, dim, ldh, heads, heads, 128, nq, nk, cos, sin, 1e-6, 0)
+        projection = dev.dev.last_kernel()
+    else:
+        lib.iris_dev_linear_bf16(h, norm, w_in, seq, dim, ldh)
+        if not q_norm_inside_attention:
+            lib.iris_dev_head_norm_rope(h, ldh, nq, cos, sin, seq, heads, 128, 1e-6, 0)
         lib.iris_dev_head_norm_rope(col(h, dim), ldh, nk, cos, sin, seq, heads, 128, 1e-6, 0)
+    if q_norm_inside_attention:
         lib.iris_dev_attention_qnorm(cat, ldc, h, col(h, dim), col(h, 2 * dim), ldh, seq, seq, heads, heads, 128, b["scale"], 0,
                                      None, nq, cos, sin, 1e-6, 0)
     else:
-        lib.iris_dev_head_norm_rope(h, ldh, nq, cos, sin, seq, heads, 128, 1e-6, 0)
-        lib.iris_dev_head_norm_rope(col(h, dim), ldh, nk, cos, sin, seq, heads, 128, 1e-6, 0)
         lib.iris_dev_attention(cat, ldc, h, col(h, dim), col(h, 2 * dim), ldh, seq, seq, heads, heads, 128, b["scale"], 0, None)
-    kernel = dev.dev.last_kernel()
+    kernel = projection or dev.dev.last_kernel()
     lib.iris_dev_swiglu(col(cat, dim), ldc, col(h, 3 * dim), col(h, 3 * dim + mlp), ldh, seq, mlp)
     lib.iris_dev_linear_f32(out, cat, w_out, seq, ldc, dim)
     lib.iris_dev_residual(x, out, ptr_add(mod, 8 * dim), seq, dim)
@@ -91,6 +96,7 @@ def test_single_stream_block_chain(dev, orc, seq, heads, mlp, backend):
     try:
         got, kernel = device_block(dev, b, False)
         fused, kernel_fused = device_block(dev, b, True)
+        one_launch, projection = device_block(dev, b, False, norm_inside_projection=True)
     finally:
         dev.lib.iris_dev_linear_backend(0)
     assert (kernel, kernel_fused) == ("fa_hd128", "fa_hd128_qnorm")
@@ -99,6 +105,12 @@ def test_single_stream_block_chain(dev, orc, seq, heads, mlp, backend):
     mx, mean = error_stats(got - b["x"], want - b["x"])
     assert mx <= 3e-2 and mean <= 3e-3, f"max-abs {mx:.4g}, mean-abs {mean:.4g}"
     assert np.array_equal(got, fused), "the block with Q normalised inside attention differs from the three-call block"
+    # the projection that normalises its own Q and K columns (rows >= 256: one launch; fewer: the two steps)
+    assert projection == ("linear_mfma_qknorm" if seq >= 256 and backend == 1 else "norm_rope_hd128")
+    mx, mean = error_stats(one_launch - b["x"], want - b["x"])
+    assert mx <= 3e-2 and mean <= 3e-3, f"projection with norm: max-abs {mx:.4g}, mean-abs {mean:.4g}"
+    if backend == 1 or projection == "norm_rope_hd128":
+        assert np.array_equal(got, one_launch), "the block with the norm inside the projection differs from the three-call block"
 
 
 # ------------------------------------------------------------------ text encoder layer (iris_qwen3.c:1586-1604)
