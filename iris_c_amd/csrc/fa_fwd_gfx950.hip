@@ -658,6 +658,314 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     }
 }
 
+/* ---- short sequences ----------------------------------------------------------------------------
+ * A workgroup of the kernel above walks its key tiles one after the other, about 1.4 us each for a wave
+ * that has its SIMD to itself, so a sequence of a few hundred keys is bound by that chain and not by the
+ * matrix cores. Here the keys of a block of 32 queries of one head are SPLIT over the S waves of a
+ * workgroup instead: wave s takes tiles s, s + S, ... (two at most up to 512 keys with S = 4), and the S
+ * partial results (running max, sum, unnormalised O^T) are merged through the LDS at the end.
+ * Nothing is shared between the waves before that, so there is no barrier in the loop and no cooperative
+ * loading: each wave loads the K tile it works on straight from global memory into the A-operand registers
+ * (16 B per lane are 8 consecutive dims of one key, which is the operand layout), and its V tile into a
+ * private 16 KB stage of the LDS (only V needs the transposing LDS read). The loads are asm statements with
+ * hand-placed waits, because two are in flight at a time and complete in order: the K tile of the next
+ * turn is requested behind this turn's QK product and the V tile behind its PV product, so "K has landed"
+ * is vmcnt <= 16 (the 16 V pieces may still be on their way) and "V has landed" likewise with the 16
+ * K loads of the turn after. Same arithmetic per tile as the kernel above. */
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+template <int S, bool CAUSAL, bool MASK>
+__global__ void __launch_bounds__(64 * S, 2)
+k_fa_short_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ q,
+                 const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
+                 int seq_q, int seq_k, int q_tiles, int kv_group, float scale_log2,
+                 const int *__restrict__ key_mask, QNorm qnorm) {
+    extern __shared__ __align__(16) uint16_t lds[];     /* S private V stages; afterwards the partial results */
+    constexpr int NB = 2, WQ = 16 * NB;
+    const int head = blockIdx.x / q_tiles;
+    int qt = blockIdx.x - head * q_tiles;
+    if (CAUSAL) qt = q_tiles - 1 - qt;             /* longest rows first */
+    const int q0 = qt * WQ;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+    const int kvh = head / kv_group;
+    const int qrow0 = q0 + li;
+    const uint16_t *kbase = k + (size_t)kvh * HD + 8 * lg;
+    const uint16_t *vbase = v + (size_t)kvh * HD;
+    uint16_t *stage = lds + wave * V_TILE;
+
+    int k_end = seq_k;
+    if (CAUSAL) k_end = min(seq_k, q0 + WQ);
+    const int ntiles = (k_end + BN - 1) / BN;
+
+    uint32_t lane_off[2];
+#pragma unroll
+    for (int par = 0; par < 2; par++)
+        lane_off[par] = (uint32_t)((lane >> 4) * ldi + 8 * ((lane & 15) ^ swz(4 * par + (lane >> 4)))) * 2u;
+
+    /* V tile `it` -> this wave's stage: 16 direct loads of 64 lanes x 16 B (four rows each). A tile that the
+     * sequence ends in redirects the missing rows to the last one (their probabilities are zero). */
+    auto request_v = [&](int it) {
+        const int kn = it * BN;
+        if (kn + BN <= seq_k) {
+            const uint16_t *src = scalar_ptr(vbase + (size_t)kn * ldi);
+            uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(stage));
+            const size_t step = 4 * (size_t)ldi;
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                             ::"s"(dst), "v"(lane_off[j & 1]), "s"(src) : "memory", "m0");
+                src += step;
+                dst += 4 * VS * 2;
+                asm volatile("" : "+s"(src), "+s"(dst));
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                const int row = 4 * j + (lane >> 4);
+                const uint16_t *src = vbase + (size_t)min(kn + row, seq_k - 1) * ldi + 8 * ((lane & 15) ^ swz(row));
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                             ::"s"(lds_address(stage + 4 * j * VS)), "v"(src) : "memory", "m0");
+            }
+        }
+    };
+    /* K tile `it` as A operands: key block mb, k-step ks -> key 16 mb + li, dims 32 ks + 8 lg .. + 7 */
+    u32x4 ka[4][4];
+    auto request_k = [&](int it) {
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) {
+            const uint16_t *kp = kbase + (size_t)min(it * BN + 16 * mb + li, seq_k - 1) * ldi;
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++)
+                asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(ka[ks][mb]) : "v"(kp), "n"(64 * ks) : "memory");
+        }
+    };
+    auto tile_mask = [&](int it) -> unsigned long long {          /* range and key mask of a tile as a 64-bit set */
+        const int key = it * BN + lane;
+        if (MASK) return __ballot(key < seq_k && key_mask[min(key, seq_k - 1)] != 0);
+        return __ballot(key < seq_k);
+    };
+
+    const bool busy = wave < ntiles;                 /* wave-uniform */
+    if (busy) request_v(wave);
+    bf16x8 qb[NB][4];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+        const uint16_t *qp = q + (size_t)min(qrow0 + 16 * nb, seq_q - 1) * ldi + (size_t)head * HD + 8 * lg;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+            qb[nb][ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 32 * ks));
+    }
+    if (busy) request_k(wave);
+    /* the masks of this wave's first two tiles here, so that the loop has no load of its own to wait for */
+    unsigned long long first_masks[2] = {~0ull, ~0ull};
+    if (MASK || k_end + BN > seq_k) {
+        first_masks[0] = tile_mask(wave);
+        first_masks[1] = tile_mask(wave + S);
+    }
+    if (qnorm.w) {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) norm_rope_q_fragment(qb[nb], qnorm, min(qrow0 + 16 * nb, seq_q - 1), lg);
+    }
+
+    int v_rd[8];
+    {
+        const int vrow = 4 * lg + (li >> 2);
+#pragma unroll
+        for (int db = 0; db < 8; db++)
+            v_rd[db] = vrow * VS + 8 * ((2 * db + ((li & 3) >> 1)) ^ swz(vrow)) + 4 * (li & 1);
+    }
+
+    const bf16x8 ones = __builtin_bit_cast(bf16x8, u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
+    f32x4 o[8][NB];
+    float m_run[NB], neg_m[NB], bound[NB];
+    f32x4 l_acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+#pragma unroll
+        for (int db = 0; db < 8; db++) o[db][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        m_run[nb] = -INFINITY; neg_m[nb] = 0.0f; bound[nb] = -INFINITY;
+        l_acc[nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    const float inv_scale_log2 = 1.0f / scale_log2;
+
+    /* Q is pinned here together with its wait (see the kernel above); the first K and V tiles, requested
+     * around it, are waited for explicitly */
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            u32x4 t = __builtin_bit_cast(u32x4, qb[nb][ks]);
+            asm volatile("" : "+v"(t));
+            qb[nb][ks] = __builtin_bit_cast(bf16x8, t);
+        }
+    wait_vmcnt<0>();
+
+    for (int it = wave, turn = 0; it < ntiles; it += S, turn++) {
+        const int k0 = it * BN;
+        const bool more = it + S < ntiles;           /* wave-uniform */
+        unsigned long long valid = ~0ull;
+        if (MASK || k0 + BN > seq_k) valid = turn < 2 ? first_masks[turn & 1] : tile_mask(it);   /* a load of the compiler's waits for everything in flight */
+
+        /* this turn's K has landed (requested before the V tile that may still be in flight) */
+        wait_vmcnt<16>();
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++) asm volatile("" : "+v"(ka[ks][mb]));
+
+        f32x4 s[4][NB];
+        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++)
+                    s[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[ks][mb]), qb[nb][ks],
+                                                                        ks == 0 ? zero : s[mb][nb], 0, 0, 0);
+        /* the operands have been read once the scores exist; only then may the registers be loaded again */
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) asm volatile("" : "+v"(s[mb][nb]));
+        if (more) request_k(it + S);
+
+        if (valid != ~0ull) {
+            const unsigned long long mine = valid >> (4 * lg);
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (!((mine >> (16 * mb + r)) & 1ull)) {
+#pragma unroll
+                        for (int nb = 0; nb < NB; nb++) s[mb][nb][r] = -INFINITY;
+                    }
+        }
+        if (CAUSAL && k0 + BN - 1 > q0) {
+            const int lim0 = qrow0 - k0 - 4 * lg;
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++)
+                        if (16 * mb + r > lim0 + 16 * nb) s[mb][nb][r] = -INFINITY;
+        }
+
+        float lane_max[NB];
+        bool raise = false;
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            const float t0 = max3(s[0][nb][0], s[0][nb][1], s[0][nb][2]), t1 = max3(s[0][nb][3], s[1][nb][0], s[1][nb][1]);
+            const float t2 = max3(s[1][nb][2], s[1][nb][3], s[2][nb][0]), t3 = max3(s[2][nb][1], s[2][nb][2], s[2][nb][3]);
+            const float t4 = max3(s[3][nb][0], s[3][nb][1], s[3][nb][2]);
+            lane_max[nb] = fmaxf(max3(t0, t1, t2), max3(t3, t4, s[3][nb][3]));
+            raise = raise || lane_max[nb] > bound[nb];
+        }
+        if (__any(raise)) {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                const float m_new = fmaxf(m_run[nb], quad_group_max(lane_max[nb]) * scale_log2);
+                const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - (m_new == -INFINITY ? 0.0f : m_new));
+                m_run[nb] = m_new;
+                neg_m[nb] = m_new == -INFINITY ? 0.0f : -m_new;
+                bound[nb] = (m_new + RESCALE_THRESHOLD) * inv_scale_log2;
+                l_acc[nb] *= alpha;
+#pragma unroll
+                for (int db = 0; db < 8; db++) o[db][nb] *= alpha;
+            }
+        }
+
+        u32x4 pw[2][NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                float p[8];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    p[r] = __builtin_amdgcn_exp2f(fmaf(s[2 * ks][nb][r], scale_log2, neg_m[nb]));
+                    p[4 + r] = __builtin_amdgcn_exp2f(fmaf(s[2 * ks + 1][nb][r], scale_log2, neg_m[nb]));
+                }
+                pw[ks][nb] = u32x4{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
+            }
+
+        /* this turn's V has landed (the next K tile, requested after it, may still be in flight) */
+        if (more) wait_vmcnt<16>(); else wait_vmcnt<0>();
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+                l_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, __builtin_bit_cast(bf16x8, pw[ks][nb]), l_acc[nb], 0, 0, 0);
+#pragma unroll
+            for (int db = 0; db < 8; db++) {
+                const uint16_t *vp = &stage[v_rd[db] + 32 * ks * VS];
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 16 * VS));
+                const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++)
+                    o[db][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), __builtin_bit_cast(bf16x8, pw[ks][nb]),
+                                                                        o[db][nb], 0, 0, 0);
+            }
+        }
+        if (more) {
+            /* every operand read of the stage has returned before it is written again */
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            request_v(it + S);
+        }
+    }
+
+    /* ---- merge the S partial results. A wave writes its O^T registers as they are over its own stage
+     * (part[wave][db][nb][lane]) and its (max, sum) behind the stages (ml[wave][nb][lane]); after the one barrier
+     * wave w merges dim blocks (8 / S) w .. : factor exp2(m_j - max_j m_j) per partial. ---- */
+    f32x4 *part = reinterpret_cast<f32x4 *>(lds);
+    float2 *ml = reinterpret_cast<float2 *>(lds + S * V_TILE);
+#pragma unroll
+    for (int db = 0; db < 8; db++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) part[((wave * 8 + db) * NB + nb) * 64 + lane] = o[db][nb];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) ml[(wave * NB + nb) * 64 + lane] = make_float2(m_run[nb], l_acc[nb][0]);
+    lds_barrier();
+    constexpr int DBS = 8 / S;
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+        float mj[S], lj[S], m_all = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < S; j++) {
+            const float2 t = ml[(j * NB + nb) * 64 + lane];
+            mj[j] = t.x; lj[j] = t.y;
+            m_all = fmaxf(m_all, t.x);
+        }
+        float l_tot = 0.0f;
+        f32x4 acc[DBS];
+#pragma unroll
+        for (int d = 0; d < DBS; d++) acc[d] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < S; j++) {
+            const float f = mj[j] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mj[j] - m_all);
+            l_tot = fmaf(f, lj[j], l_tot);
+#pragma unroll
+            for (int d = 0; d < DBS; d++) acc[d] += f * part[((j * 8 + DBS * wave + d) * NB + nb) * 64 + lane];
+        }
+        const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+        const int qrow = qrow0 + 16 * nb;
+        if (qrow < seq_q) {
+            uint16_t *op = out + (size_t)qrow * ldo + (size_t)head * HD + 4 * lg;
+#pragma unroll
+            for (int d = 0; d < DBS; d++) {
+                uint2 w;
+                w.x = pack_bf16(acc[d][0] * inv, acc[d][1] * inv);
+                w.y = pack_bf16(acc[d][2] * inv, acc[d][3] * inv);
+                *reinterpret_cast<uint2 *>(op + 16 * (DBS * wave + d)) = w;
+            }
+        }
+    }
+}
+#pragma clang diagnostic pop
+
 template <int W, int NB> constexpr size_t stage_bytes() { return (W * NB >= 12 ? 4 : 2) * STAGE * sizeof(uint16_t); }
 constexpr size_t LDS_MAX = 160 * 1024;
 constexpr int CUS = 256;
@@ -697,6 +1005,34 @@ int launch_w(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const ui
     return launch<W, NB, false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
 }
 
+template <int S, bool C, bool M>
+int launch_short(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi,
+                 int seq_q, int seq_k, int heads, int kv_heads, float scale, const int *key_mask, const QNorm &qn) {
+    static bool configured = false;
+    constexpr size_t lds_bytes = (size_t)S * (V_TILE * sizeof(uint16_t) + 1024);     /* stages / partial O^T, and (max, sum) */
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_short_hd128<S, C, M>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+        configured = true;
+    }
+    const int q_tiles = (seq_q + 31) / 32;
+    hipLaunchKernelGGL((k_fa_short_hd128<S, C, M>), dim3(heads * q_tiles), dim3(64 * S), lds_bytes, st, out, ldo,
+                       q, k, v, ldi, seq_q, seq_k, q_tiles, heads / kv_heads, scale * 1.4426950408889634f, key_mask, qn);
+    return (int)hipGetLastError();
+}
+
+template <int S>
+int launch_short_cm(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi,
+                    int seq_q, int seq_k, int heads, int kv_heads, float scale, int causal, const int *key_mask, const QNorm &qn) {
+    if (causal) {
+        if (key_mask) return launch_short<S, true, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
+        return launch_short<S, true, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
+    }
+    if (key_mask) return launch_short<S, false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
+    return launch_short<S, false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn);
+}
+
 }  // namespace
 
 static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
@@ -712,6 +1048,21 @@ static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16
      * none does (one wave per SIMD runs faster than two, not twice as fast). Constants measured on
      * 24 heads, 256 .. 12800 tokens, clocks settled. */
     const long units = (long)((seq_q + 31) / 32) * heads;          /* waves of 32 queries */
+    /* Few workgroups and more than one key tile: the keys of a query block are split over the waves of a
+     * workgroup (k_fa_short_hd128). Measured against the choices below, clocks settled, rows in the L2:
+     * 24 heads x 320 tokens 9.0 us against 10.5, x 256 7.5 against 9.1, 1 head x 512 9.0 against 14.3,
+     * 8 heads x 1024 15.0 against 23.0, 2 heads x 1000 causal + mask 14.2 against 30.4. With more than one
+     * workgroup per CU (32 heads x 512 tokens: 512) the private tiles cost what the shorter chain saves
+     * (a CU then pulls 320 KB through its 64 B / clock L1 port): 16.4 against 16.9 us, left where it was. */
+    {
+        const long q_tiles32 = (seq_q + 31) / 32;
+        const long keys = causal ? (seq_k < 32 * q_tiles32 ? seq_k : 32 * q_tiles32) : seq_k;
+        const long tiles = (keys + BN - 1) / BN;
+        if (tiles >= 2 && q_tiles32 * heads <= CUS) {
+            if (tiles >= 6) return launch_short_cm<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+            return launch_short_cm<2>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+        }
+    }
     if (units >= 576) {
         const long wg256 = (long)((seq_q + 255) / 256) * heads, wg128 = (long)((seq_q + 127) / 128) * heads;
         const long cost8 = 100 * ((wg256 + CUS - 1) / CUS);

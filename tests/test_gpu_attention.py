@@ -115,13 +115,15 @@ def test_c2_full_size_sampled_rows_and_properties(dev, orc):
 
 
 @pytest.mark.parametrize("seq,heads,kv,causal,masked", [
-    (200, 6, 6, False, False), (200, 6, 2, True, True),              # 32-query workgroups (one wave)
+    (200, 6, 6, False, False), (200, 6, 2, True, True),              # keys split over two waves (four key tiles)
+    (40, 40, 10, False, False), (60, 48, 12, True, True),            # one key tile: 32-query workgroups (one wave)
     (600, 16, 4, False, True), (600, 16, 16, True, False),           # 64-query workgroups
     (1300, 16, 16, False, False), (1300, 16, 8, True, True),         # 128-query workgroups
     (2100, 24, 8, False, True), (2100, 24, 24, True, False),         # 256-query workgroups
 ])
 def test_every_workgroup_width(dev, orc, seq, heads, kv, causal, masked):
-    """The launcher picks 32, 64, 128 or 256 queries per workgroup from the problem size; each
+    """The launcher picks 32, 64, 128 or 256 queries per workgroup from the problem size (or, for few workgroups
+    and several key tiles, the kernel that splits the keys over the waves); each
     width is its own instantiation of the kernel (pieces of a key tile per wave, LDS stages).
     Sampled rows against the oracle, including the rows around every workgroup boundary."""
     rng = np.random.default_rng(seq + heads)
@@ -207,6 +209,44 @@ def test_c3_full_size_masked_equals_compacted(dev, orc, fa):
 
 
 # ------------------------------------------------------------------ edge cases
+@pytest.mark.parametrize("seq_q,seq_k,heads,kv,causal,masked", [
+    (77, 333, 8, 2, False, True),          # six key tiles over four waves: two waves take two tiles
+    (40, 130, 3, 3, False, False),         # three tiles over two waves
+    (500, 500, 4, 2, True, True),          # causal: the waves of the first query blocks have no tile at all
+    (1000, 1000, 2, 2, True, True),        # four tiles per wave: the masks of the later ones are read in the loop
+    (33, 3000, 1, 1, False, True),         # twelve turns per wave, ragged last tile
+    (512, 512, 8, 8, False, False),        # 128 workgroups x 4 waves
+])
+def test_keys_split_over_the_waves_of_a_workgroup(dev, orc, seq_q, seq_k, heads, kv, causal, masked):
+    """Few (head, 32-query block) pairs and more than one key tile: every wave of a workgroup takes every S-th
+    key tile of the same queries and the partial results are merged at the end. All rows against the oracle."""
+    rng = np.random.default_rng(seq_q + seq_k)
+    buf, ldi = random_case(seq_q * 3 + seq_k, seq_q, seq_k, heads, kv)
+    qd, kd = heads * 128, kv * 128
+    mask = None
+    if masked:
+        mask = (rng.random(seq_k) < 0.7).astype(np.int32)
+        mask[0] = 1
+        mask[64:128] = 0                       # a whole tile without a valid key: that wave's partial result is empty
+    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, 128, 0.0884, causal, mask)
+    assert kernel == "fa_hd128"
+    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, 128, 0.0884, causal, mask)
+    assert_close(O.bf16_to_f32(out[:seq_q]), want, f"{seq_q}x{seq_k} heads {heads}/{kv} causal={causal} masked={masked}")
+
+
+def test_split_keys_with_rows_that_have_no_valid_key(dev, orc):
+    """Rows whose every key is masked give zeros from the merge as well (all partial maxima are -inf)."""
+    seq, heads = 300, 2
+    buf, ldi = random_case(9, seq, seq, heads, heads)
+    mask = np.zeros(seq, np.int32)
+    mask[200:] = 1                               # causal rows 0 .. 199 see no valid key
+    out, kernel = dev.attention(buf, ldi, 0, heads * 128, 2 * heads * 128, seq, seq, heads, heads, 128, 0.0884, True, mask)
+    got = O.bf16_to_f32(out)
+    assert np.all(got[:200] == 0.0) and np.isfinite(got).all()
+    want = orc.attention_bf16(buf, ldi, 0, heads * 128, 2 * heads * 128, seq, seq, heads, heads, 128, 0.0884, True, mask)
+    assert_close(got[200:], want[200:], "rows behind the empty ones")     # (the fp32 CPU attention has no zero-row rule)
+
+
 def random_case(seed, seq_q, seq_k, heads, kv_heads, hd=128, pad=0, sigma=1.0):
     rng = np.random.default_rng(seed)
     seq = max(seq_q, seq_k)
