@@ -58,6 +58,21 @@ def traffic_on_file():
         pass
     return None, None
 
+NORM_ROPE_PROFILE = os.path.join("profiles", "k_norm_rope_hd128__c2__kernel_trace.txt")
+
+
+def kernel_only_on_file():
+    """Kernel-only durations (us) of the norm+rope series from the committed kernel trace: lines 'name: value'."""
+    found = {}
+    try:
+        for line in open(os.path.join(ROOT, NORM_ROPE_PROFILE)):
+            for name in ("q_call_kernel_us_cold", "qk_fused_kernel_us_cold", "q_call_kernel_us_warm"):
+                if line.startswith(name + ":"):
+                    found[name] = float(line.split(":")[1])
+    except (OSError, ValueError):
+        pass
+    return found
+
 _vp = C.c_void_p
 
 
@@ -692,10 +707,10 @@ def main():
                       "warm_cache_q_call_us": round(nr_warm_ms * 1e3, 2),
                       "warm_cache_q_call_frac": round(q_bytes / (nr_warm_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
                       "q_call_single_launch_us": round(single_launch_ms(hip, stream, lib, res.norm_q) * 1e3, 2),
+                      "kernel_only_us_on_file": kernel_only_on_file(), "kernel_only_source": NORM_ROPE_PROFILE,
                       "note": "cold = 8 rotating 85 MB row buffers (> 256 MB Infinity Cache); warm = same buffer every call; "
-                              "averages over back-to-back launches between two events. In a kernel trace of the same series "
-                              "consecutive launches abut, so these are also the kernel-only durations "
-                              "(profiles/k_norm_rope_hd128__c2__kernel_trace.txt)"},
+                              "averages over back-to-back launches between two events. kernel_only_us_on_file: the kernel-only "
+                              "durations of the same three series in the committed kernel trace (a separate profiler run)"},
     }
     res.free()
 
