@@ -8,19 +8,43 @@
  * A wave cannot hold a 512-wide output row block in registers, so the head
  * dimension is cut into NS slices of 128 and a group of NS waves shares 32
  * queries: wave (g, s) keeps Q[:, 128s .. 128s+127] and O[:, same] of group
- * g's queries. For every tile of 32 keys each wave multiplies its slice,
- *     S_part^T = K[:, slice] Q[:, slice]^T        (8 MFMAs 32x32x16),
- * the NS partial score blocks are exchanged through LDS and added in slice
- * order, so every wave of the group holds bit-identical scores and runs the
- * same online softmax redundantly; then O[:, slice]^T += V[:, slice]^T P^T
- * (8 MFMAs). As in the 128 kernel both products are transposed, a lane owns
- * one query, and exp2(S^T) in bf16 is directly the B operand.
+ * g's queries. Workgroup = 8 waves = 8/NS query groups (64 queries at 512,
+ * 128 at 256). For every tile of 32 keys
+ *   A  each wave multiplies its slice, S_part^T = K[:, slice] Q[:, slice]^T
+ *      (8 MFMAs 32x32x16), and leaves the partial scores in the LDS;
+ *   B  the keys of the tile are dealt out to the NS waves of the group (8 each
+ *      at 512): a wave adds the NS partial scores of ITS keys only, so the
+ *      softmax is done once per group and not once per wave. The running max
+ *      of a query is shared by the group: every wave publishes the largest of
+ *      its 8 scores per query, all read the NS maxima and take the same
+ *      decision (the max is only raised, and the accumulators rescaled, when a
+ *      score exceeds it by more than 2^8). Then exp2 of the own keys, rounded
+ *      to bf16, goes to the LDS in the layout of the B operand;
+ *   C  every wave reads the whole P^T of the tile and adds
+ *      O[:, slice]^T += V[:, slice]^T P^T (8 MFMAs).
+ * Three barriers per tile (partial scores, maxima, probabilities). As in the
+ * 128 kernel both products are transposed and a lane owns one query. The row
+ * sum of a query is kept per wave over its own keys and added up at the end.
  *
- * Workgroup = 8 waves = 8/NS query groups (64 queries at 512, 128 at 256).
- * One LDS stage [K tile 32 x (HD+8) | V tile 32 x (HD+32)] plus the exchange
- * area; the next tile waits in registers while the current one is used.
- * Three barriers per tile: scores exchanged / tile consumed / next tile
- * stored.
+ * K and V tiles have two LDS stages each (K two tiles ahead, V one) and are
+ * fetched a further tile ahead into registers. Rows are unpadded; the 16 B
+ * chunk c of row r sits in slot c ^ sw(r) of its 256 B group,
+ * sw(r) = 4 (r % 4) + (r / 4) % 4: the 16 rows of a ds_read_b128 pass land in
+ * 16 different slots, and the four rows of a transposing read in four
+ * different 64 B windows.
+ *
+ * Where the time goes (16384 tokens x 1 head x 512, 0.90-0.93 ms, 24 % of the
+ * bf16 matrix peak): a tile of 32 keys takes about 4000 cycles per wave, the
+ * sum of a chain of dependent steps, each an LDS round trip of about 350
+ * cycles or a chain of eight products that wait for one another (570): K
+ * operands, partial scores out and in, maxima out and in, probabilities out
+ * and in, V operands; the two waves of a SIMD are in the same step at the same
+ * time (the barriers), so they do not fill each other's waits. What does NOT
+ * bound it, each tried with the rest unchanged: the tile loads (direct loads,
+ * register-staged loads or none at all: 0.90-0.93 ms), the second or the third
+ * barrier (removed, wrong results: 0.90), the softmax arithmetic (done once
+ * per wave instead of once per group: 0.93), two accumulator chains in the
+ * score product (0.94). The K/V tiles come from the L2 (96 % hits).
  */
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -52,12 +76,6 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2));
 }
 
-__device__ __forceinline__ float max3(float a, float b, float c) {
-    float d;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
-    return d;
-}
-
 __device__ __forceinline__ float half_swap_max(float v) {
     auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
@@ -66,6 +84,10 @@ __device__ __forceinline__ float half_swap_sum(float v) {
     auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+
+__device__ __forceinline__ int sw(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+/* slot of chunk c (16 B) of tile row r */
+__device__ __forceinline__ int slot_of(int c, int row) { return (c & ~15) | ((c ^ sw(row)) & 15); }
 
 template <int NS, bool CAUSAL, bool MASK>
 __global__ void __launch_bounds__(THREADS, 2)
@@ -76,15 +98,15 @@ k_fa_fwd_sliced(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict_
     constexpr int HD = 128 * NS;
     constexpr int QG = 8 / NS;             /* query groups per workgroup */
     constexpr int BM = 32 * QG;
-    constexpr int KS = HD + 8;             /* K tile row stride in elements: 16 B x odd */
-    constexpr int VS = HD + 32;            /* V tile row stride: 64 B x odd */
-    constexpr int K_TILE = BN * KS, V_TILE = BN * VS;
-    constexpr int CPR = HD / 8;            /* 16 B chunks per row */
-    constexpr int NP = BN * CPR / THREADS; /* chunks of K (and of V) per thread and tile = NS */
-    constexpr int RSTEP = THREADS / CPR;   /* rows between a thread's chunks */
+    constexpr int TILE = BN * HD;          /* elements of a K (or V) tile */
+    constexpr int CH = HD / 8;             /* 16 B chunks per row */
+    constexpr int OWN = 4 / NS;            /* blocks of 8 keys a wave owns in a tile */
+    constexpr int SLOTS = NS == 4 ? 3 : 4; /* blocks of partial scores a wave leaves for the others (at 512 its own one stays in registers) */
 
-    extern __shared__ __align__(16) uint16_t lds[];     /* [K tile | V tile | score exchange] */
-    f32x4 *xch = reinterpret_cast<f32x4 *>(lds + K_TILE + V_TILE);   /* [QG][NS][4][64] */
+    extern __shared__ __align__(16) uint16_t lds[];     /* K stage 0, 1 | V stage 0, 1 | partial scores | P^T | maxima */
+    f32x4 *x1 = reinterpret_cast<f32x4 *>(lds + 4 * TILE);            /* [8 waves][SLOTS][64 lanes] */
+    uint16_t *x2 = reinterpret_cast<uint16_t *>(x1 + 8 * SLOTS * 64);  /* [QG][2 k-steps][2][32 queries][8] */
+    float *x3 = reinterpret_cast<float *>(x2 + QG * 4 * 32 * 8);       /* [8 waves][32 queries] */
 
     const int work = (blockIdx.x % XCDS) * work_per_xcd + blockIdx.x / XCDS;
     if (work >= total_work) return;
@@ -93,13 +115,48 @@ k_fa_fwd_sliced(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict_
     if (CAUSAL) qt = q_tiles - 1 - qt;
     const int kvh = head / kv_group;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int sl = wave % NS, grp = wave / NS;
     const int col = lane & 31, hh = lane >> 5;
     const int q0 = qt * BM, wq0 = q0 + grp * 32, qrow = wq0 + col;
 
     const uint16_t *kbase = k + (size_t)kvh * HD;
     const uint16_t *vbase = v + (size_t)kvh * HD;
+
+    int k_end = seq_k;
+    if (CAUSAL) k_end = min(seq_k, q0 + BM);
+    const int ntiles = (k_end + BN - 1) / BN;
+    const int last_k0 = (ntiles - 1) * BN;
+
+    /* ---- tile loads. A thread moves NS chunks of 16 B of a K tile and of a V tile: rows row0 + RSTEP c, chunk
+     * tid % CH. They wait in registers for a whole tile period (global load -> ds_write one turn later): issuing a
+     * direct global -> LDS load costs a wave about 100 cycles each here, eight of them a tile, on the critical path. */
+    constexpr int NP = NS, RSTEP = THREADS / CH;
+    const int row0 = tid / CH, cchunk = tid % CH;
+    u32x4 tk[NP], tv[NP];
+    auto fetch_k = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < NP; c++)
+            tk[c] = *reinterpret_cast<const u32x4 *>(kbase + (size_t)min(k0 + row0 + RSTEP * c, seq_k - 1) * ldi + 8 * cchunk);
+    };
+    auto fetch_v = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < NP; c++)
+            tv[c] = *reinterpret_cast<const u32x4 *>(vbase + (size_t)min(k0 + row0 + RSTEP * c, seq_k - 1) * ldi + 8 * cchunk);
+    };
+    int st_off[NP];                         /* where the thread's chunks go inside a stage (elements) */
+#pragma unroll
+    for (int c = 0; c < NP; c++) st_off[c] = (row0 + RSTEP * c) * HD + 8 * slot_of(cchunk, row0 + RSTEP * c);
+    auto store = [&](uint16_t *stage, const u32x4 (&t)[NP]) {
+#pragma unroll
+        for (int c = 0; c < NP; c++) *reinterpret_cast<u32x4 *>(&stage[st_off[c]]) = t[c];
+    };
+    uint16_t *kst = lds, *vst = lds + 2 * TILE;
+    fetch_k(0); fetch_v(0);
+    store(kst, tk); store(vst, tv);
+    fetch_k(min(BN, last_k0));
+    store(kst + TILE, tk);
+    fetch_k(min(2 * BN, last_k0)); fetch_v(min(BN, last_k0));      /* wait in registers for the first turn */
 
     /* This wave's slice of Q^T as B operands: dims 128 sl + 16t + 8hh .. +7. */
     bf16x8 qb[8];
@@ -114,105 +171,111 @@ k_fa_fwd_sliced(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict_
     for (int db = 0; db < 4; db++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;     /* l_run: over this wave's keys only */
 
-    int k_end = seq_k;
-    if (CAUSAL) k_end = min(seq_k, q0 + BM);
-    const int ntiles = (k_end + BN - 1) / BN;
-    const int last_k0 = (ntiles - 1) * BN;
-
-    /* LDS read addresses (elements): K operand row = key `col`, 16 B at dims 128 sl + 16t + 8hh;
-     * V^T operand through the transpose read, rows 4hh + (lane%16)/4 (+16t, +8),
-     * columns 128 sl + 16 ((lane/16)%2) + 4 (lane%4) (+32 db). */
-    const int k_rd = col * KS + 128 * sl + 8 * hh;
-    const int v_rd = K_TILE + (4 * hh + ((lane & 15) >> 2)) * VS + 128 * sl + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-
-    /* This thread's chunks of a tile: rows row0 + RSTEP c, 16 B at element column ccol. */
-    const int row0 = tid / CPR, ccol = (tid % CPR) * 8;
-    u32x4 tk[NP], tv[NP];
-    auto fetch = [&](int k0) {
+    /* LDS read offsets (elements, relative to a stage). K operand of k-step t: row = key `col`, chunk 16 sl + 2t + hh.
+     * V^T operand (k-step t of 16 keys, dim block db, half hi): transposing read of rows 16t + 8hi + 4hh + (lane%16)/4,
+     * 8 B at chunk 16 sl + 4 db + 2 ((lane/16)%2) + (lane%4)/2, element 4 (lane%2) inside it. */
+    int k_rd[8], v_rd[2][4];
 #pragma unroll
-        for (int c = 0; c < NP; c++) {
-            const int r = min(k0 + row0 + RSTEP * c, seq_k - 1);     /* rows past the end: masked later */
-            const size_t off = (size_t)r * ldi + ccol;
-            tk[c] = *reinterpret_cast<const u32x4 *>(kbase + off);
-            tv[c] = *reinterpret_cast<const u32x4 *>(vbase + off);
-        }
-    };
-    auto store = [&]() {
+    for (int t = 0; t < 8; t++) k_rd[t] = col * HD + 8 * slot_of(16 * sl + 2 * t + hh, col);
 #pragma unroll
-        for (int c = 0; c < NP; c++) {
-            const int r = row0 + RSTEP * c;
-            *reinterpret_cast<u32x4 *>(&lds[r * KS + ccol]) = tk[c];
-            *reinterpret_cast<u32x4 *>(&lds[K_TILE + r * VS + ccol]) = tv[c];
+    for (int hi = 0; hi < 2; hi++)
+#pragma unroll
+        for (int db = 0; db < 4; db++) {
+            const int row = 8 * hi + 4 * hh + ((lane & 15) >> 2);      /* + 16 t: sw(row) does not change with t */
+            v_rd[hi][db] = row * HD + 8 * slot_of(16 * sl + 4 * db + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), row) + 4 * (lane & 1);
         }
-    };
 
-    fetch(0);
-    store();
-    fetch(min(BN, last_k0));
-    __syncthreads();
+    lds_barrier();
 
     for (int it = 0; it < ntiles; it++) {
         const int k0 = it * BN;
+        const uint16_t *kcur = kst + (it & 1) * TILE, *vcur = vst + (it & 1) * TILE;
 
-        /* ---- partial scores over this wave's 128 dims ---- */
+        /* ---- A: partial scores over this wave's 128 dims ---- */
         f32x16 s;
         {
             u32x4 ka[8];
 #pragma unroll
-            for (int t = 0; t < 8; t++) ka[t] = *reinterpret_cast<const u32x4 *>(&lds[k_rd + 16 * t]);
+            for (int t = 0; t < 8; t++) ka[t] = *reinterpret_cast<const u32x4 *>(&kcur[k_rd[t]]);
             const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
             s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[0]), qb[0], zero, 0, 0, 0);
 #pragma unroll
             for (int t = 1; t < 8; t++)
                 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[t]), qb[t], s, 0, 0, 0);
         }
-        /* ---- exchange: every wave of the group adds the NS parts in slice order ---- */
-        {
-            f32x4 *mine = xch + ((grp * NS + sl) * 4) * 64 + lane;
+        /* register r holds key k0 + 8 (r/4) + 4 hh + r%4 for query qrow: block r/4 of 8 keys. This wave owns blocks
+         * OWN sl .. ; the others go to the LDS for their owners. */
 #pragma unroll
-            for (int g = 0; g < 4; g++) mine[g * 64] = f32x4{s[4 * g], s[4 * g + 1], s[4 * g + 2], s[4 * g + 3]};
-            lds_barrier();
-            const f32x4 *all = xch + (grp * NS * 4) * 64 + lane;
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                f32x4 a = all[g * 64];
-#pragma unroll
-                for (int p = 1; p < NS; p++) a += all[(p * 4 + g) * 64];
-                s[4 * g] = a.x; s[4 * g + 1] = a.y; s[4 * g + 2] = a.z; s[4 * g + 3] = a.w;
-            }
+        for (int g = 0; g < 4; g++) {
+            if (NS == 4 && g == sl) continue;
+            const int slot = NS == 4 ? (g < sl ? g : g - 1) : g;
+            x1[(wave * SLOTS + slot) * 64 + lane] = f32x4{s[4 * g], s[4 * g + 1], s[4 * g + 2], s[4 * g + 3]};
         }
-        /* register r holds key k0 + 8(r/4) + 4hh + r%4 for query qrow */
+        lds_barrier();                                                       /* 1: partial scores */
+        /* K stage (it % 2) and V stage ((it + 1) % 2) have no readers any more: K of tile it + 2 and V of tile it + 1
+         * go there from the registers, and the loads of the turn after are issued */
+        store(kst + (it & 1) * TILE, tk);
+        store(vst + ((it + 1) & 1) * TILE, tv);
+        fetch_k(min(k0 + 3 * BN, last_k0));
+        fetch_v(min(k0 + 2 * BN, last_k0));
 
-        /* ---- validity ---- */
+        f32x4 mine[OWN];
+#pragma unroll
+        for (int ob = 0; ob < OWN; ob++) {
+            const int g = OWN * sl + ob;
+            f32x4 a = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int p = 0; p < NS; p++) {                                   /* in slice order */
+                if (p == sl) {
+                    f32x4 own;
+                    /* block g of this wave's registers; g is wave-uniform but not a constant: selected without indexing */
+#pragma unroll
+                    for (int gg = 0; gg < 4; gg++)
+                        if (gg == g) own = f32x4{s[4 * gg], s[4 * gg + 1], s[4 * gg + 2], s[4 * gg + 3]};
+                    a += own;
+                } else {
+                    const int slot = NS == 4 ? (g < p ? g : g - 1) : g;
+                    a += x1[((grp * NS + p) * SLOTS + slot) * 64 + lane];
+                }
+            }
+            mine[ob] = a;
+        }
+
+        /* ---- validity of the own keys: key k0 + 8 (OWN sl + ob) + 4 hh + r ---- */
         unsigned valid = ~0u;
         if (k0 + BN > seq_k) valid = (1u << (seq_k - k0)) - 1u;
         if (MASK) {
             const unsigned long long b = __ballot(lane < BN && (k0 + lane < seq_k) && key_mask[min(k0 + lane, seq_k - 1)] != 0);
             valid &= (unsigned)b;
         }
-        if (valid != ~0u) {
-            const unsigned mine = valid >> (4 * hh);
 #pragma unroll
-            for (int r = 0; r < 16; r++)
-                if (!((mine >> (8 * (r >> 2) + (r & 3))) & 1u)) s[r] = -INFINITY;
+        for (int ob = 0; ob < OWN; ob++) {
+            const int kin = 8 * (OWN * sl + ob) + 4 * hh;                    /* first of the lane's four keys, inside the tile */
+            if (valid != ~0u) {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (!((valid >> (kin + r)) & 1u)) mine[ob][r] = -INFINITY;
+            }
+            if (CAUSAL && k0 + BN - 1 > wq0) {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (k0 + kin + r > qrow) mine[ob][r] = -INFINITY;
+            }
         }
-        if (CAUSAL && k0 + BN - 1 > wq0) {
-            const int lim = qrow - k0 - 4 * hh;
+        float mx = -INFINITY;
 #pragma unroll
-            for (int r = 0; r < 16; r++)
-                if (8 * (r >> 2) + (r & 3) > lim) s[r] = -INFINITY;
-        }
-
-        /* ---- online softmax, one query per lane ---- */
-        float mx = max3(s[0], s[1], s[2]);
+        for (int ob = 0; ob < OWN; ob++) mx = fmaxf(mx, fmaxf(fmaxf(mine[ob][0], mine[ob][1]), fmaxf(mine[ob][2], mine[ob][3])));
+        mx = half_swap_max(mx);
+        if (hh == 0) x3[wave * 32 + col] = mx;
+        lds_barrier();                                                       /* 2: maxima */
+        float tile_max = x3[(grp * NS) * 32 + col];
 #pragma unroll
-        for (int r = 3; r < 15; r += 2) mx = max3(mx, s[r], s[r + 1]);
-        mx = fmaxf(mx, s[15]);
-        mx = half_swap_max(mx) * scale_log2;
-        if (__any(mx > m_run + RESCALE_THRESHOLD)) {
-            const float m_new = fmaxf(m_run, mx);
+        for (int p = 1; p < NS; p++) tile_max = fmaxf(tile_max, x3[(grp * NS + p) * 32 + col]);
+        tile_max *= scale_log2;
+        if (__any(tile_max > m_run + RESCALE_THRESHOLD)) {                   /* the same decision in every wave of the group */
+            const float m_new = fmaxf(m_run, tile_max);
             const float alpha = __builtin_amdgcn_exp2f(m_run - (m_new == -INFINITY ? 0.0f : m_new));
             m_run = m_new;
             l_run *= alpha;
@@ -222,47 +285,54 @@ k_fa_fwd_sliced(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict_
                 for (int r = 0; r < 16; r++) o[db][r] *= alpha;
         }
         const float neg_m = m_run == -INFINITY ? 0.0f : -m_run;
-        float psum = 0.0f;
-        uint32_t pw[8];                            /* pw[4t + j]: k-step t, elements 2j, 2j+1 */
 #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-            const float p0 = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2, neg_m));
-            const float p1 = __builtin_amdgcn_exp2f(fmaf(s[r + 1], scale_log2, neg_m));
-            psum += p0 + p1;
-            pw[r >> 1] = pack_bf16(p0, p1);
+        for (int ob = 0; ob < OWN; ob++) {
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(mine[ob][0], scale_log2, neg_m));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(mine[ob][1], scale_log2, neg_m));
+            const float p2 = __builtin_amdgcn_exp2f(fmaf(mine[ob][2], scale_log2, neg_m));
+            const float p3 = __builtin_amdgcn_exp2f(fmaf(mine[ob][3], scale_log2, neg_m));
+            l_run += (p0 + p1) + (p2 + p3);
+            /* P^T in the layout of the B operand, [k-step t of 16 keys][hh][query][8]: the lane (query, hh) of the product
+             * multiplies keys 16t + 4hh + 0..3 and 16t + 8 + 4hh + 0..3 (the rows its V^T operand brings), i.e. this
+             * lane's four keys of block 2t or 2t + 1 */
+            const int kb = OWN * sl + ob;
+            *reinterpret_cast<uint2 *>(&x2[((((grp * 2) + (kb >> 1)) * 2 + hh) * 32 + col) * 8 + 4 * (kb & 1)]) =
+                make_uint2(pack_bf16(p0, p1), pack_bf16(p2, p3));
         }
-        l_run += psum;
+        lds_barrier();                                                       /* 3: probabilities; V of this tile, K of the next */
 
-        /* ---- O[:, slice]^T += V[:, slice]^T P^T ---- */
+        /* ---- C: O[:, slice]^T += V[:, slice]^T P^T ---- */
         {
+            bf16x8 pb[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+                pb[t] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(&x2[((((grp * 2) + t) * 2 + hh) * 32 + col) * 8]));
             s16x4 lo[2][4], hi[2][4];
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
                 for (int db = 0; db < 4; db++) {
-                    const uint16_t *vp = &lds[v_rd + 16 * t * VS + 32 * db];
-                    lo[t][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp));
-                    hi[t][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 8 * VS));
+                    lo[t][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(&vcur[v_rd[0][db] + 16 * t * HD]));
+                    hi[t][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(&vcur[v_rd[1][db] + 16 * t * HD]));
                 }
 #pragma unroll
-            for (int t = 0; t < 2; t++) {
-                uint4 praw = make_uint4(pw[4 * t], pw[4 * t + 1], pw[4 * t + 2], pw[4 * t + 3]);
-                bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
+            for (int t = 0; t < 2; t++)
 #pragma unroll
                 for (int db = 0; db < 4; db++) {
                     s16x8 both = __builtin_shufflevector(lo[t][db], hi[t][db], 0, 1, 2, 3, 4, 5, 6, 7);
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pb, o[db], 0, 0, 0);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pb[t], o[db], 0, 0, 0);
                 }
-            }
         }
-        lds_barrier();                              /* tile and exchange area consumed by every wave */
-        store();                                    /* tile it+1 */
-        fetch(min(k0 + 2 * BN, last_k0));           /* tile it+2 */
-        lds_barrier();
     }
-
-    /* ---- normalise and store this wave's 128 dims: lane holds dims 32db + 8g + 4hh + {0..3} ---- */
-    const float l_tot = half_swap_sum(l_run);
+    /* ---- the row sums of the NS waves of a group, then normalise and store this wave's 128 dims:
+     * lane holds dims 32db + 8g + 4hh + {0..3} ---- */
+    lds_barrier();
+    const float l_wave = half_swap_sum(l_run);
+    if (hh == 0) x3[wave * 32 + col] = l_wave;
+    lds_barrier();
+    float l_tot = x3[(grp * NS) * 32 + col];
+#pragma unroll
+    for (int p = 1; p < NS; p++) l_tot += x3[(grp * NS + p) * 32 + col];
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
     if (qrow < seq_q) {
         uint16_t *op = out + (size_t)qrow * ldo + (size_t)head * HD + 128 * sl + 4 * hh;
@@ -283,7 +353,9 @@ int launch(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint
            const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads, float scale,
            const int *key_mask) {
     constexpr int HD = 128 * NS, BM = 32 * (8 / NS);
-    constexpr size_t LDS_BYTES = (size_t)(BN * (HD + 8) + BN * (HD + 32)) * sizeof(uint16_t) + 8 * 4 * 64 * sizeof(f32x4);
+    /* two K and two V stages, partial scores (8 waves x 3 or 4 blocks x 1 KB), P^T, maxima */
+    constexpr size_t LDS_BYTES = (size_t)4 * BN * HD * sizeof(uint16_t) + (size_t)8 * (NS == 4 ? 3 : 4) * 64 * sizeof(f32x4) +
+                                 (size_t)(8 / NS) * 4 * 32 * 8 * sizeof(uint16_t) + 8 * 32 * sizeof(float);
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_sliced<NS, C, M>),
