@@ -21,9 +21,27 @@ CFLAGS   = -O2 -fPIC -Wall -Wextra -std=c11 $(HOSTDEFS) -I$(CSRC) -Iinclude -I$(
 HIP_SRCS = $(CSRC)/qknorm_rope.hip $(CSRC)/fa_fwd_gfx950.hip $(CSRC)/fa_fwd_sliced_gfx950.hip $(CSRC)/attn_generic.hip \
            $(CSRC)/ew_norm_ops.hip $(CSRC)/gemm_conv_gfx950.hip $(CSRC)/rope_tables.hip
 HIP_OBJS = $(HIP_SRCS:.hip=.o)
+HOST_HDRS = include/iris_dev.h include/iris_rope.h $(CSRC)/iris_kernels_hip.h $(CSRC)/iris_rope_internal.h
 
-.PHONY: rocm oracle clean test-cpu test-gpu bench ctest
+.PHONY: rocm oracle clean test-cpu test-gpu bench ctest path pathcheck
 rocm: $(OUT) iris_c_amd/libiris_microbench.so
+
+# The hot path alone, for a host backend that keeps everything else (its own init, memory entries, stream and the
+# other operators): the attention and norm+rope kernels and their two dispatch functions, none of the setup /
+# memory / operator symbols that would clash with the host's.
+PATH_LIB = iris_c_amd/libiris_dev_path.a
+path: $(PATH_LIB)
+$(CSRC)/iris_rocm_path.o: $(CSRC)/iris_rocm.c $(HOST_HDRS)
+	$(CC) $(CFLAGS) -DIRIS_DEV_PATH_ONLY -c $< -o $@
+$(PATH_LIB): $(CSRC)/qknorm_rope.o $(CSRC)/fa_fwd_gfx950.o $(CSRC)/fa_fwd_sliced_gfx950.o $(CSRC)/attn_generic.o $(CSRC)/iris_rocm_path.o
+	rm -f $@ && ar rcs $@ $^
+# link check: a host program that defines its OWN iris_dev_init / alloc / ... (as the reference's backend object
+# does) next to the archive: no duplicate symbols, the hot-path calls resolve to the archive
+pathcheck: tests/path_only_link.bin
+tests/path_only_link.bin: tests/path_only_link.c include/iris_dev.h include/iris_dev_path.h $(PATH_LIB)
+	$(CC) -O2 -Wall -Wextra -std=c11 $(HOSTDEFS) -Iinclude -I$(ROCM_HOME)/include -c $< -o tests/path_only_link.o
+	$(HIPCC) --offload-arch=$(GPU_ARCH) -o $@ tests/path_only_link.o $(PATH_LIB) -L$(ROCM_HOME)/lib -lamdhip64 -lm \
+	    -Wl,-rpath,$(ROCM_HOME)/lib
 
 # C-language parity program: host C over the ABI, checked against the oracle (run by the GPU tests)
 ctest: tests/c_abi_parity.bin
@@ -41,7 +59,6 @@ iris_c_amd/libiris_microbench.so: $(CSRC)/microbench.hip
 $(CSRC)/%.o: $(CSRC)/%.hip $(CSRC)/iris_kernels_hip.h $(CSRC)/norm_rope_math.h
 	$(HIPCC) $(HIPFLAGS) -c $< -o $@
 
-HOST_HDRS = include/iris_dev.h include/iris_rope.h $(CSRC)/iris_kernels_hip.h $(CSRC)/iris_rope_internal.h
 $(CSRC)/iris_rocm.o: $(CSRC)/iris_rocm.c $(HOST_HDRS)
 	$(CC) $(CFLAGS) -c $< -o $@
 
@@ -67,4 +84,4 @@ bench:
 	python bench.py
 
 clean:
-	rm -f $(CSRC)/*.o $(OUT) iris_c_amd/libiris_microbench.so tests/c_abi_parity.bin
+	rm -f $(CSRC)/*.o $(OUT) $(PATH_LIB) iris_c_amd/libiris_microbench.so tests/c_abi_parity.bin tests/path_only_link.bin tests/path_only_link.o

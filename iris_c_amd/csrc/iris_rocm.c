@@ -29,19 +29,23 @@ static int g_last_error = 0;
 static const char *g_last_kernel = "none";
 /* private scratch, allocated on first use and kept until cleanup (as the reference backend
  * does, iris_cuda.cu:149-173): convolution patches and group-norm partial sums */
+#ifndef IRIS_DEV_PATH_ONLY
 #define CONV_SCRATCH_BYTES ((size_t)256 << 20)
 static uint16_t *g_conv_scratch = NULL;
 static float *g_gn_scratch = NULL;
 static size_t g_gn_scratch_floats = 0;
+#endif
 /* normalised copy of Q for the iris_dev_attention_qnorm calls that the matrix-core kernel does not take */
 static uint16_t *g_q_scratch = NULL;
 static size_t g_q_scratch_bytes = 0;
 /* padded, aligned copy of q | k | v (and the padded output) for attention calls on other head sizes or alignments */
 static uint16_t *g_pack = NULL;
 static size_t g_pack_bytes = 0;
+#ifndef IRIS_DEV_PATH_ONLY
 /* staging buffer of the rotary tables being expanded: column map, row offsets, dictionary */
 static void *g_rope_stage = NULL;
 static size_t g_rope_stage_bytes = 0;
+#endif
 
 static void fail(int code, const char *what, const char *detail) {
     g_last_error = code ? code : -1;
@@ -60,6 +64,7 @@ static int need_ready(const char *what) {
     return 0;
 }
 
+#ifndef IRIS_DEV_PATH_ONLY
 int iris_dev_init(void) {
     if (g_ready) return 1;
     int count = 0;
@@ -84,9 +89,13 @@ int iris_dev_init(void) {
     return 1;
 }
 
+#endif
+
+#ifndef IRIS_DEV_PATH_ONLY
 int iris_dev_available(void) { return g_ready; }
 const char *iris_dev_name(void) { return g_name; }
 void *iris_dev_stream(void) { return (void *)g_stream; }
+#endif
 const char *iris_dev_last_kernel(void) { return g_last_kernel; }
 
 int iris_dev_last_error(void) {
@@ -95,6 +104,7 @@ int iris_dev_last_error(void) {
     return e;
 }
 
+#ifndef IRIS_DEV_PATH_ONLY
 void iris_dev_cleanup(void) {
     if (!g_ready) return;
     check(hipStreamSynchronize(g_stream), "sync");
@@ -158,6 +168,30 @@ void iris_dev_sync(void) {
     if (!need_ready("sync")) return;
     check(hipStreamSynchronize(g_stream), "sync");
 }
+
+#else
+/* Path-only build (libiris_dev_path.a): the two hot-path operators for a host backend that keeps its own setup,
+ * memory entries and stream. The host attaches the stream its other work runs on; the operators enqueue there. */
+void iris_dev_path_attach(void *hip_stream) {
+    (void)g_name;
+    g_stream = (hipStream_t)hip_stream;
+    g_ready = 1;
+    g_last_error = 0;
+}
+
+void iris_dev_path_detach(void) {
+    if (!g_ready) return;
+    check(hipStreamSynchronize(g_stream), "sync");
+    if (g_q_scratch) check(hipFree(g_q_scratch), "free");
+    if (g_pack) check(hipFree(g_pack), "free");
+    g_q_scratch = NULL;
+    g_q_scratch_bytes = 0;
+    g_pack = NULL;
+    g_pack_bytes = 0;
+    g_stream = NULL;
+    g_ready = 0;
+}
+#endif
 
 static int aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
@@ -334,6 +368,7 @@ void iris_dev_attention_qnorm(uint16_t *out, int ldo,
 
 /* ---- the other operators: thin checked wrappers over the launchers ---- */
 
+#ifndef IRIS_DEV_PATH_ONLY
 #define LAUNCH(what, call)                                        \
     do {                                                          \
         if (!need_ready(what)) return;                            \
@@ -625,3 +660,4 @@ void iris_dev_rope_qwen3_tables(float *d_cos, float *d_sin, const int *attention
     rope_tables("rope_qwen3_tables", d_cos, d_sin, pos, seq, 1, &head_dim, NULL, theta, 0);
     free(pos);
 }
+#endif /* !IRIS_DEV_PATH_ONLY */

@@ -100,6 +100,22 @@ def test_unmodified_reference_links_against_this_backend(lib):
     assert "libiris_dev.so" in ldd and "not found" not in ldd
 
 
+def test_path_only_archive_links_next_to_a_host_backend():
+    """libiris_dev_path.a (the hot path for a host that keeps its own backend): defines the two operators, their
+    additions and attach / detach, none of the setup / memory / other-operator symbols, and links into a program
+    that defines those itself (tests/path_only_link.c)."""
+    import subprocess
+    subprocess.check_call(["make", "-s", "-C", ROOT, "path", "pathcheck"], stderr=subprocess.DEVNULL)
+    out = subprocess.run(["nm", "--defined-only", os.path.join(ROOT, "iris_c_amd", "libiris_dev_path.a")],
+                         capture_output=True, text=True, check=True).stdout
+    defined = {line.split()[-1] for line in out.splitlines() if " T iris_dev_" in line}
+    assert defined == {"iris_dev_head_norm_rope", "iris_dev_head_norm_rope_qk", "iris_dev_attention", "iris_dev_attention_qnorm",
+                       "iris_dev_last_error", "iris_dev_last_kernel", "iris_dev_path_attach", "iris_dev_path_detach"}
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "iris_dev_path.h")).read(), flags=re.S)
+    assert set(re.findall(r"\b(iris_dev_\w+)\s*\(", text)) == {"iris_dev_path_attach", "iris_dev_path_detach"}
+    assert os.path.exists(os.path.join(ROOT, "tests", "path_only_link.bin"))
+
+
 def test_division_constant_of_the_norm_rope_kernel(lib):
     """The fast norm+rope kernel turns a unit index into (token, head) with one multiply-high by
     the constant its launcher computes (0 = "one head, no division"). Checked the way the kernel

@@ -35,3 +35,14 @@ def test_c_program_parity_on_gpu():
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "all checks passed" in r.stdout and "kernel: fa_sliced" in r.stdout
+
+
+@pytest.mark.gpu
+def test_path_only_archive_runs_behind_a_host_backend():
+    """tests/path_only_link.c: a host program with its own init / memory entries / stream, linked against
+    libiris_dev_path.a, normalises Q and K and runs attention over a constant V: every output must be that constant."""
+    exe = os.path.join(ROOT, "tests", "path_only_link.bin")
+    if not os.path.exists(exe):
+        subprocess.check_call(["make", "-s", "-C", ROOT, "path", "pathcheck"])
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0 and r.stdout.startswith("ok (fa_hd128)"), r.stdout + r.stderr
