@@ -6,18 +6,30 @@ sequence: fused per-head RMSNorm + RoPE on Q, on K, then joint attention
 (reference iris_transformer_flux.c:3834-3839), on the 24 heads x 128,
 512 text + 4096 image token configuration, bf16, inputs resident in HBM.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle-ms T] [--no-cpu] [--no-shapes]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle-ms T] [--no-cpu] [--no-shapes] [--no-machine]
+    python bench.py --only CONFIG [--steps K]     launches of one configuration only (C1 .. C5, C3-cond, C3-uncond,
+                                                  VAE), for profiler runs
+    python bench.py --copy-only MiB               the plain copy kernel that calibrates the byte counters
 
 Prints ONE JSON line. `value` is attention TFLOP/s over the whole step
-(algorithmic attention FLOPs / wall time of the triple). `roofline` is the
-attention kernel alone, timed with HIP events on the library's stream around
-the attention launch of every step. `norm_rope` reports the bandwidth-bound
-kernel over back-to-back launches. `shapes` lists
-latency / TFLOP/s / GB/s for every benchmark configuration, `other_ops` the
-other device operators at this configuration's shapes, `rope_tables` the
-time to build one forward pass's rotary tables (host builder + upload, and
-the device generator). `cpu_baseline`
-times the reference's BLAS-build CPU structure on this host's cores.
+(algorithmic attention FLOPs / wall time of the triple) with settled clocks,
+`value_from_idle` the same over the first 50 steps after the GPU sat idle.
+`roofline` is the attention kernel alone, timed with HIP events on the
+library's stream around the attention launch of every step (mean, median,
+min, and the latency of a single launch between two synchronisations); its
+`traffic` is read from the committed counter summary it names. `norm_rope`
+reports the bandwidth-bound kernel over back-to-back launches (cold rows,
+fused Q+K, rows in the Infinity Cache) and the kernel-only durations on file.
+`shapes` lists, for every benchmark configuration, the attention latency
+(mean / median / min / single launch) with its fraction of the matrix peak,
+the norm+rope calls with their fraction of the HBM peak, and the seconds of
+the CPU port on this host's cores; `other_ops` the other device operators
+at this configuration's shapes, among them the q | k | v projection with
+and without the normalisation in its epilogue; `rope_tables` the time to
+build one forward pass's rotary tables (host builder + upload, and straight
+into device memory); `machine` the measured ceilings of the GPU and the
+attention kernel by number of busy CUs. `cpu_baseline` times the
+reference's BLAS-build CPU structure on this host's cores.
 
 Clock settling: after idle the GPU's power management takes tens of
 milliseconds of sustained load to reach its steady clocks; the same
