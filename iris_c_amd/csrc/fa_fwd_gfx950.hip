@@ -17,16 +17,18 @@
  *
  * Shape of the computation on CDNA4
  * ---------------------------------
- * One workgroup = WAVES (8, 4, 2 or 1) waves of 32 queries of one head; each
- * wave owns its 32 queries for the whole kernel. 8 waves = 256 queries is the
- * throughput shape (two waves share a SIMD, one workgroup per CU); the smaller
- * ones are taken when the problem has too few queries to give every CU a
- * large workgroup: a workgroup walks its key tiles one after the other, so a
- * short sequence is bound by that latency and wants many small workgroups.
+ * One workgroup = WAVES (8, 4, 2 or 1) waves of NB blocks of 16 queries of one
+ * head; each wave owns its queries for the whole kernel. 8 waves x 32 queries
+ * (NB = 2) = 256 queries is the throughput shape (two waves share a SIMD, one
+ * workgroup per CU), 4 x 32 the alternative for the large problems whose
+ * rounds over the CUs it fills better. A workgroup walks its key tiles one
+ * after the other, so a short sequence is bound by that latency: problems of
+ * up to 2048 waves of 16 queries take NB = 1, as many small workgroups as it
+ * takes to fill the CUs (or the kernel further down that splits the keys).
  * Keys/values stream through LDS in tiles of 64 keys, 4 stages (2 below 8
- * waves), and they go there directly: global_load_lds_dwordx4 copies
+ * waves of 32 queries), and they go there directly: global_load_lds_dwordx4 copies
  * HBM/L2 -> LDS without passing through registers, one group of tiles
- * (two tiles, one below 8 waves) ahead of the group in use; one barrier per
+ * (two tiles, one with the smaller shapes) ahead of the group in use; one barrier per
  * group. Every wave reads the whole K and V tile,
  * so 256 queries per workgroup mean half the L2 -> LDS traffic per query of
  * 128.
@@ -1038,43 +1040,54 @@ int launch_short_cm(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, c
 static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
                             const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads, float scale,
                             int causal, const int *key_mask, const QNorm &qn) {
-    /* A workgroup walks its key tiles one after the other, about 2 us each, so a short sequence is
-     * bound by that latency and wants many small workgroups: 32 or 64 queries when the larger
-     * shapes would leave CUs without work. From 576 waves of 32 queries on, the choice is between
-     * 256 queries (8 waves, one workgroup fills a CU, half the K/V traffic from L2 per query) and
-     * 128 queries (4 waves, two workgroups per CU), by the cost of their rounds over the 256 CUs,
-     * in units of one full round of 256-query workgroups: such a round costs 1 however few CUs it
-     * uses; a round of 128-query workgroups costs 1.13 when some CU gets two of them and 0.72 when
-     * none does (one wave per SIMD runs faster than two, not twice as fast). Constants measured on
-     * 24 heads, 256 .. 12800 tokens, clocks settled. */
-    const long units = (long)((seq_q + 31) / 32) * heads;          /* waves of 32 queries */
-    /* Few workgroups and more than one key tile: the keys of a query block are split over the waves of a
-     * workgroup (k_fa_short_hd128). Measured against the choices below, clocks settled, rows in the L2:
-     * 24 heads x 320 tokens 9.0 us against 10.5, x 256 7.5 against 9.1, 1 head x 512 9.0 against 14.3,
-     * 8 heads x 1024 15.0 against 23.0, 2 heads x 1000 causal + mask 14.2 against 30.4. With more than one
-     * workgroup per CU (32 heads x 512 tokens: 512) the private tiles cost what the shorter chain saves
-     * (a CU then pulls 320 KB through its 64 B / clock L1 port): 16.4 against 16.9 us, left where it was. */
-    {
+    /* Three regimes, by the number of waves of 16 queries the problem makes (heads x ceil(seq_q / 16)).
+     *
+     * Up to 2048 of them (one wave per SIMD and CU slot, or fewer): a workgroup walks its key tiles one after the
+     * other, so a short sequence is bound by that chain, and the chain is shortest when a wave carries ONE block
+     * of 16 queries (NB = 1: half the products per tile and wave, twice the waves): 1, 2, 4 or 8 such waves per
+     * workgroup so that the workgroups about fill the 256 CUs. Measured, clocks settled, rows in the L2, against
+     * 32 queries per wave: 32 heads on 8 x 512 tokens causal + mask 11.9 us against 15.5; 24 heads x 320 tokens
+     * 7.7 against 10.5, x 576 11.8 against 15.2, x 768 17.4 against 20.2, x 1280 26.0 against 29.8 (x 1536: 56 against
+     * 45, the other way round); same bits either way. About 0.65 us per key tile with up to two waves per
+     * workgroup, 0.92 with four, 1.08 with eight.
+     * When the (head, 32-query block) pairs are at most one per CU and the sequence has many key tiles, splitting
+     * the keys over the waves of a workgroup (k_fa_short_hd128) is shorter still: 1.45 us per turn of
+     * ceil(tiles / S) plus 1.5 for the merge. 1 head x 512 tokens 9.0 us against 9.8; 8 heads x 1024 14.9 against
+     * 16.9; 4 heads x 2000 + mask 25.4 against 32.5. (With more than one workgroup per CU its private tiles cost
+     * what the shorter chain saves: 32 heads x 512 tokens, 512 workgroups, 16.4 us.)
+     *
+     * Beyond that, 32 queries per wave, and the choice is between 256 queries (8 waves, one workgroup fills a CU,
+     * half the K/V traffic from L2 per query) and 128 queries (4 waves, two workgroups per CU), by the cost of
+     * their rounds over the 256 CUs, in units of one full round of 256-query workgroups: such a round costs 1
+     * however few CUs it uses; a round of 128-query workgroups costs 1.13 when some CU gets two of them and 0.72
+     * when none does (one wave per SIMD runs faster than two, not twice as fast). Constants measured on 24 heads,
+     * 256 .. 12800 tokens, clocks settled. */
+    const long waves16 = (long)((seq_q + 15) / 16) * heads;
+    if (waves16 <= 8 * CUS) {
+        const int w = waves16 <= CUS ? 1 : waves16 <= 640 ? 2 : waves16 <= 4 * CUS ? 4 : 8;
         const long q_tiles32 = (seq_q + 31) / 32;
         const long keys = causal ? (seq_k < 32 * q_tiles32 ? seq_k : 32 * q_tiles32) : seq_k;
         const long tiles = (keys + BN - 1) / BN;
+        const long cost_chain = tiles * (w <= 2 ? 65 : w == 4 ? 92 : 108);           /* 0.01 us */
         if (tiles >= 2 && q_tiles32 * heads <= CUS) {
-            if (tiles >= 6) return launch_short_cm<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
-            return launch_short_cm<2>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+            const int s = tiles >= 6 ? 4 : 2;
+            if (((tiles + s - 1) / s) * 145 + 150 < cost_chain) {
+                if (s == 4) return launch_short_cm<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+                return launch_short_cm<2>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+            }
         }
+        if (w == 1) return launch_w<1, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+        if (w == 2) return launch_w<2, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+        if (w == 4) return launch_w<4, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+        return launch_w<8, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
     }
-    if (units >= 576) {
-        const long wg256 = (long)((seq_q + 255) / 256) * heads, wg128 = (long)((seq_q + 127) / 128) * heads;
-        const long cost8 = 100 * ((wg256 + CUS - 1) / CUS);
-        const long rest4 = wg128 % (2 * CUS);
-        const long cost4 = 113 * (wg128 / (2 * CUS)) + (rest4 == 0 ? 0 : rest4 <= CUS ? 72 : 113);
-        if (cost8 <= cost4)
-            return launch_w<8>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
-        return launch_w<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
-    }
-    if (units >= 256)
-        return launch_w<2>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
-    return launch_w<1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+    const long wg256 = (long)((seq_q + 255) / 256) * heads, wg128 = (long)((seq_q + 127) / 128) * heads;
+    const long cost8 = 100 * ((wg256 + CUS - 1) / CUS);
+    const long rest4 = wg128 % (2 * CUS);
+    const long cost4 = 113 * (wg128 / (2 * CUS)) + (rest4 == 0 ? 0 : rest4 <= CUS ? 72 : 113);
+    if (cost8 <= cost4)
+        return launch_w<8>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+    return launch_w<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
 }
 
 extern "C" int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uint16_t *q,

@@ -115,16 +115,18 @@ def test_c2_full_size_sampled_rows_and_properties(dev, orc):
 
 
 @pytest.mark.parametrize("seq,heads,kv,causal,masked", [
-    (200, 6, 6, False, False), (200, 6, 2, True, True),              # keys split over two waves (four key tiles)
-    (40, 40, 10, False, False), (60, 48, 12, True, True),            # one key tile: 32-query workgroups (one wave)
-    (600, 16, 4, False, True), (600, 16, 16, True, False),           # 64-query workgroups
-    (1300, 16, 16, False, False), (1300, 16, 8, True, True),         # 128-query workgroups
-    (2100, 24, 8, False, True), (2100, 24, 24, True, False),         # 256-query workgroups
+    (200, 6, 6, False, False), (200, 6, 2, True, True),              # 78 waves of 16 queries: one-wave workgroups
+    (40, 40, 10, False, False), (60, 48, 12, True, True),            # one key tile
+    (330, 24, 24, False, False), (300, 24, 8, True, True),           # two waves of 16 queries per workgroup
+    (600, 16, 4, False, True), (600, 16, 16, True, False),           # four
+    (1300, 16, 16, False, False), (1300, 16, 8, True, True),         # eight
+    (2100, 24, 8, False, True), (2100, 24, 24, True, False),         # 32 queries per wave: 128- or 256-query workgroups
+    (4200, 8, 8, False, False), (1500, 24, 24, False, True),
 ])
 def test_every_workgroup_width(dev, orc, seq, heads, kv, causal, masked):
-    """The launcher picks 32, 64, 128 or 256 queries per workgroup from the problem size (or, for few workgroups
-    and several key tiles, the kernel that splits the keys over the waves); each
-    width is its own instantiation of the kernel (pieces of a key tile per wave, LDS stages).
+    """The launcher picks the workgroup from the problem size: 1, 2, 4 or 8 waves of 16 queries for up to 2048 such
+    waves, 4 or 8 waves of 32 queries beyond (or, for few workgroups and many key tiles, the kernel that splits the
+    keys over the waves); each shape is its own instantiation of the kernel (pieces of a key tile per wave, LDS stages).
     Sampled rows against the oracle, including the rows around every workgroup boundary."""
     rng = np.random.default_rng(seq + heads)
     ldi = (heads + 2 * kv) * 128
