@@ -22,8 +22,9 @@ reports the bandwidth-bound kernel over back-to-back launches (cold rows,
 fused Q+K, rows in the Infinity Cache) and the kernel-only durations on file.
 `shapes` lists, for every benchmark configuration, the attention latency
 (mean / median / min / single launch) with its fraction of the matrix peak,
-the norm+rope calls with their fraction of the HBM peak, and the seconds of
-the CPU port on this host's cores; `other_ops` the other device operators
+the norm+rope calls with their fraction of the HBM peak, the whole step
+(two norm+rope calls and attention) issued call by call and replayed from a
+HIP graph of 16 steps, and the seconds of the CPU port on this host's cores; `other_ops` the other device operators
 at this configuration's shapes, among them the q | k | v projection with
 and without the normalisation in its epilogue; `rope_tables` the time to
 build one forward pass's rotary tables (host builder + upload, and straight
@@ -168,6 +169,23 @@ class Hip:
         assert self.rt.hipEventElapsedTime(C.byref(ms), a, b) == 0
         return float(ms.value)
 
+    def capture(self, stream, fn):
+        """Records what fn enqueues on the library's stream into a graph; returns the executable graph."""
+        rt = self.rt
+        rt.hipStreamBeginCapture.argtypes = [_vp, C.c_int]
+        rt.hipStreamEndCapture.argtypes = [_vp, C.POINTER(_vp)]
+        rt.hipGraphInstantiate.argtypes = [C.POINTER(_vp), _vp, _vp, _vp, C.c_size_t]
+        rt.hipGraphLaunch.argtypes = [_vp, _vp]
+        rt.hipGraphExecDestroy.argtypes = [_vp]
+        rt.hipGraphDestroy.argtypes = [_vp]
+        assert rt.hipStreamBeginCapture(stream, 0) == 0
+        fn()
+        graph, run = _vp(), _vp()
+        assert rt.hipStreamEndCapture(stream, C.byref(graph)) == 0 and graph
+        assert rt.hipGraphInstantiate(C.byref(run), graph, None, None, 0) == 0
+        rt.hipGraphDestroy(graph)
+        return run
+
 
 class Resident:
     """One configuration's tensors in HBM, `copies` rotating row buffers."""
@@ -261,6 +279,31 @@ def single_launch_ms(hip, stream, lib, fn, reps=5):
         hip.record(a, stream); fn(i); hip.record(b, stream)
         ts.append(hip.elapsed_ms(a, b))
     return float(np.median(ts))
+
+
+def step_times(hip, stream, lib, step, steps_per_graph=16, launches=8):
+    """(eager, graph) microseconds per step: the caller's triple issued call by call, and the same steps captured
+    once into a HIP graph of `steps_per_graph` steps and replayed (what a launch-bound loop such as the layers of the
+    text encoder would do; the library's operators allocate nothing, so its stream can be captured)."""
+    n = steps_per_graph * launches
+    for i in range(steps_per_graph):
+        step(i)
+    lib.iris_dev_sync()
+    t0 = time.perf_counter()
+    for i in range(n):
+        step(i)
+    lib.iris_dev_sync()
+    eager = (time.perf_counter() - t0) / n * 1e6
+    run = hip.capture(stream, lambda: [step(i) for i in range(steps_per_graph)])
+    assert hip.rt.hipGraphLaunch(run, stream) == 0
+    lib.iris_dev_sync()
+    t0 = time.perf_counter()
+    for _ in range(launches):
+        assert hip.rt.hipGraphLaunch(run, stream) == 0
+    lib.iris_dev_sync()
+    graph = (time.perf_counter() - t0) / n * 1e6
+    hip.rt.hipGraphExecDestroy(run)
+    return eager, graph
 
 
 def per_launch_times(hip, stream, fn, reps, before=None):
@@ -753,6 +796,8 @@ def main():
                      "norm_rope_q_frac_of_hbm_peak": round(qb / q_ms / 1e6 / PEAK_HBM_GBPS, 4),
                      "norm_rope_qk_us": round(qk_ms * 1e3, 2), "norm_rope_qk_gbps": round(nb / qk_ms / 1e6, 1),
                      "norm_rope_qk_frac_of_hbm_peak": round(nb / qk_ms / 1e6 / PEAK_HBM_GBPS, 4)}
+            eager_us, graph_us = step_times(hip, stream, lib, r.step)
+            entry.update(step_us=round(eager_us, 2), step_us_in_hip_graph=round(graph_us, 2))
             dev.check()
             r.free()
             if not args.no_cpu:

@@ -1,0 +1,74 @@
+"""The hot path under HIP graph capture. The library enqueues on one stream that it hands out
+(iris_dev_stream), and the two hot-path operators allocate nothing, so a caller can capture a
+step -- norm+rope on Q, on K, attention -- into a graph once and replay it (what a launch-bound loop
+such as the 36 layers of the text encoder wants). Every replay is checked against the eager result,
+with eager work and synchronisations of the program between the replays.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import workloads as W
+from gpu_harness import Dev, ptr_add
+
+pytestmark = pytest.mark.gpu
+_vp = C.c_void_p
+
+
+class Graphs:
+    def __init__(self):
+        self.rt = C.CDLL("libamdhip64.so")
+        self.rt.hipStreamBeginCapture.argtypes = [_vp, C.c_int]
+        self.rt.hipStreamEndCapture.argtypes = [_vp, C.POINTER(_vp)]
+        self.rt.hipGraphInstantiate.argtypes = [C.POINTER(_vp), _vp, _vp, _vp, C.c_size_t]
+        self.rt.hipGraphLaunch.argtypes = [_vp, _vp]
+        self.rt.hipGraphExecDestroy.argtypes = [_vp]
+        self.rt.hipGraphDestroy.argtypes = [_vp]
+
+    def capture(self, stream, fn):
+        assert self.rt.hipStreamBeginCapture(stream, 0) == 0          # hipStreamCaptureModeGlobal
+        fn()
+        graph, run = _vp(), _vp()
+        assert self.rt.hipStreamEndCapture(stream, C.byref(graph)) == 0 and graph
+        assert self.rt.hipGraphInstantiate(C.byref(run), graph, None, None, 0) == 0
+        self.rt.hipGraphDestroy(graph)
+        return run
+
+
+@pytest.mark.parametrize("maker", [W.c1, W.c4, lambda: W.c2(shrink=4)], ids=["c1", "c4", "c2-shrunk"])
+def test_step_replayed_from_a_graph_equals_the_eager_step(maker):
+    case = maker()
+    dev, g = Dev(), Graphs()
+    lib, stream = dev.lib, _vp(dev.lib.iris_dev_stream())
+    seq, ldi, qd, kd = case["seq"], case["ldi"], case["q_dim"], case["kv_dim"]
+    rows, out = dev.put(case["buf"]), dev.alloc(seq * case["ldo"] * 2)
+    wq, wk, cos, sin = dev.put(case["wq"]), dev.put(case["wk"]), dev.put(case["cos"]), dev.put(case["sin"])
+    mask = dev.put(np.ascontiguousarray(case["key_mask"], np.int32)) if case["key_mask"] is not None else None
+
+    def step():
+        lib.iris_dev_head_norm_rope(rows, ldi, wq, cos, sin, seq, case["heads"], 128, case["eps"], case["split_half"])
+        lib.iris_dev_head_norm_rope(ptr_add(rows, 2 * qd), ldi, wk, cos, sin, seq, case["kv_heads"], 128, case["eps"], case["split_half"])
+        lib.iris_dev_attention(out, case["ldo"], rows, ptr_add(rows, 2 * qd), ptr_add(rows, 2 * (qd + kd)), ldi, seq, seq,
+                               case["heads"], case["kv_heads"], 128, case["scale"], int(case["causal"]), mask)
+
+    step()                                              # eager (also the first launch of each kernel: attributes are set here)
+    dev.check()
+    want = dev.get(out, (seq, case["ldo"]), np.uint16)
+    assert want.any()
+    run = g.capture(stream, step)
+    dev.check()
+    host = np.ascontiguousarray(case["buf"])
+    for replay in range(4):
+        # eager work of the program between the replays: the rows are normalised in place, so they are uploaded again,
+        # and the output is overwritten with a pattern
+        lib.iris_dev_upload(rows, host.ctypes.data_as(_vp), host.nbytes)
+        junk = np.full((seq, case["ldo"]), 0x7fc0 + replay, np.uint16)
+        lib.iris_dev_upload(out, junk.ctypes.data_as(_vp), junk.nbytes)
+        assert g.rt.hipGraphLaunch(run, stream) == 0
+        lib.iris_dev_sync()
+        dev.check()
+        got = dev.get(out, (seq, case["ldo"]), np.uint16)
+        assert np.array_equal(got, want), f"replay {replay} differs from the eager step"
+    g.rt.hipGraphExecDestroy(run)
+    dev.free_all()
