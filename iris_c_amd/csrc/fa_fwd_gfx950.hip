@@ -449,11 +449,24 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     wait_vmcnt<0>();
     lds_barrier();                                       /* also publishes the key-mask words */
 
-    for (int g0 = 0, half = 0; g0 < ntiles; g0 += GROUP, half ^= 1) {
+    /* Key tiles behind the last one that holds a valid key change nothing (their probabilities are all
+     * zero), so the walk ends there: a prompt of 40 tokens padded to 512 costs one tile, not eight. Every
+     * wave reads the same words and gets the same count, which the barriers in the loop rely on. */
+    int ntiles_run = ntiles;
+    if (MASK) {
+        while (ntiles_run > 0) {
+            const unsigned long long word = mask_words[ntiles_run - 1];
+            const uint32_t any = __builtin_amdgcn_readfirstlane((uint32_t)word | (uint32_t)(word >> 32));
+            if (any) break;
+            ntiles_run--;
+        }
+    }
+
+    for (int g0 = 0, half = 0; g0 < ntiles_run; g0 += GROUP, half ^= 1) {
 #pragma unroll
       for (int h = 0; h < GROUP; h++) {
         const int it = g0 + h;
-        if (it >= ntiles) break;                         /* wave-uniform */
+        if (it >= ntiles_run) break;                     /* wave-uniform */
         const int k0 = it * BN;
         uint16_t *cur = lds + (half * GROUP + h) * STAGE;
 

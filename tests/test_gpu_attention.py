@@ -144,6 +144,26 @@ def test_every_workgroup_width(dev, orc, seq, heads, kv, causal, masked):
     assert_close(got[rows], cpu_attention(orc, case, rows=rows), f"seq {seq} heads {heads}/{kv}")
 
 
+@pytest.mark.parametrize("seq,heads,kv,causal,valid", [
+    (512, 32, 8, True, 40), (512, 32, 8, True, 1), (512, 32, 8, False, 65),        # a short prompt padded to 512
+    (2100, 24, 8, False, 130), (2100, 24, 24, True, 700), (4608, 24, 24, False, 4113),
+])
+def test_padding_behind_the_last_valid_key_is_not_walked(dev, orc, seq, heads, kv, causal, valid):
+    """A key mask that is a prefix (a prompt padded to a fixed length): the kernel stops at the last key tile that
+    holds a valid key. Same results as the oracle, which walks every key; padded query rows included."""
+    rng = np.random.default_rng(seq + valid)
+    ldi = (heads + 2 * kv) * 128
+    buf = O.f32_to_bf16(rng.standard_normal((seq, ldi)).astype(np.float32))
+    mask = (np.arange(seq) < valid).astype(np.int32)
+    case = W._case(buf=buf, heads=heads, kv_heads=kv, causal=causal, key_mask=mask)
+    case["ldo"] = heads * 128
+    got, kernel = gpu_attention(dev, case)
+    assert kernel == "fa_hd128"
+    rows = np.unique(np.r_[sample_rows(seq, n=24, seed=valid), [valid - 1, valid % seq, 63, 64]]).astype(np.int32)
+    rows = rows[(rows >= 0) & (rows < seq)]
+    assert_close(got[rows], cpu_attention(orc, case, rows=rows), f"seq {seq}, {valid} valid keys")
+
+
 def test_very_long_masked_key_sequence_takes_the_generic_kernel(dev, orc):
     """The matrix-core kernel keeps the key mask in LDS, one bit per key, which bounds a masked
     seq_k at 250000; beyond that the call must still be answered (by the generic kernel)."""
