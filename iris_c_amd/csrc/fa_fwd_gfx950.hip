@@ -25,6 +25,11 @@
  * after the other, so a short sequence is bound by that latency: problems of
  * up to 2048 waves of 16 queries take NB = 1, as many small workgroups as it
  * takes to fill the CUs (or the kernel further down that splits the keys).
+ * The waves of a workgroup need not carry the same number of blocks: when the
+ * last round of 256-query workgroups would leave CUs idle (432 workgroups on
+ * 256 CUs run as 256 + 176), the last queries of every head go to workgroups
+ * of 192 queries, four waves of 32 and four of 16, so that the last round
+ * uses every CU for about 0.78 of a full round (k_fa_fwd_hd128_two_sizes).
  * Keys/values stream through LDS in tiles of 64 keys, 4 stages (2 below 8
  * waves of 32 queries), and they go there directly: global_load_lds_dwordx4 copies
  * HBM/L2 -> LDS without passing through registers, one group of tiles
@@ -98,8 +103,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
-/* A workgroup is WAVES waves of NB blocks of 16 queries (NB = 2 in every launch): BM = 16 * NB * WAVES queries,
- * 64 * WAVES threads. */
 constexpr int BN = 64;             /* keys per tile */
 constexpr int HD = 128;
 constexpr int KS = HD;              /* K and V tile rows are 256 B, unpadded: chunks are swizzled instead */
@@ -318,35 +321,21 @@ __device__ __forceinline__ void norm_rope_q_fragment(bf16x8 (&qb)[4], const QNor
 }
 
 
-template <int WAVES, int NB, bool CAUSAL, bool MASK>
-__global__ void __launch_bounds__(64 * WAVES, 2)
-k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ q,
-               const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
-               int seq_q, int seq_k, int q_tiles, int total_work, int work_per_xcd,
-               int kv_group, float scale_log2, const int *__restrict__ key_mask, QNorm qnorm) {
-    extern __shared__ __align__(16) uint16_t lds[];     /* NSTAGE stages of [K tile | V tile] */
-    constexpr int WQ = 16 * NB;                          /* queries per wave: NB blocks of 16 */
-    constexpr int BM = WQ * WAVES, NI = (32 + WAVES - 1) / WAVES;   /* pieces of a tile per wave (the last waves may have one fewer) */
-    /* Key tiles between two barriers. Two for the 8-wave shape (one workgroup per CU, so the LDS
-     * has room for four stages): the waves of a workgroup then only meet every other tile, and
-     * the faster ones do not stand at a barrier while the slower ones finish every single tile. */
-    constexpr int GROUP = WAVES * NB >= 12 ? 2 : 1;
+/* The walk of one wave over the key tiles of its workgroup. WAVES and GROUP belong to the workgroup (pieces of a
+ * tile per wave, tiles between two barriers, stages); NB, the blocks of 16 queries the wave carries, may differ
+ * between the waves of a workgroup as long as every wave passes the same barriers: the tile count depends on the
+ * workgroup's queries q0 .. q0 + bm - 1 only. wq0 is the wave's first query. */
+template <int WAVES, int NB, int GROUP, bool CAUSAL, bool MASK>
+__device__ __forceinline__ void
+fa_walk_hd128(uint16_t *__restrict__ lds, uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ q,
+              const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
+              int seq_q, int seq_k, int head, int kvh, int q0, int bm, int wq0,
+              float scale_log2, const int *__restrict__ key_mask, const QNorm &qnorm) {
+    constexpr int NI = (32 + WAVES - 1) / WAVES;         /* pieces of a tile per wave (the last waves may have one fewer) */
     constexpr int NSTAGE = 2 * GROUP;                    /* the group in use and the group on its way */
-
-    /* XCD-aware numbering: hardware deals workgroups round-robin to the 8
-     * XCDs, so id%8 is the XCD; give each XCD a contiguous slice of the
-     * head-major work list. */
-    const int work = (blockIdx.x % XCDS) * work_per_xcd + blockIdx.x / XCDS;
-    if (work >= total_work) return;
-    const int head = work / q_tiles;
-    int qt = work - head * q_tiles;
-    if (CAUSAL) qt = q_tiles - 1 - qt;             /* longest rows first */
-    const int q0 = qt * BM;
-    const int kvh = head / kv_group;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;       /* 16x16 block: column li, row group lg */
-    const int wq0 = q0 + wave * WQ;
     const int qrow0 = wq0 + li;                     /* this lane's queries: qrow0 + 16 nb, one per query block */
 
     const uint16_t *kbase = k + (size_t)kvh * HD;
@@ -357,7 +346,7 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     const bf16x8 ones = __builtin_bit_cast(bf16x8, u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
 
     int k_end = seq_k;
-    if (CAUSAL) k_end = min(seq_k, q0 + BM);       /* keys beyond the last query of the block are never valid */
+    if (CAUSAL) k_end = min(seq_k, q0 + bm);       /* keys beyond the last query of the workgroup are never valid */
     const int ntiles = (k_end + BN - 1) / BN;
 
     /* LDS read addresses (elements, relative to a stage).
@@ -671,6 +660,75 @@ k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             }
         }
     }
+}
+
+/* Workgroups of WAVES waves that all carry NB blocks of 16 queries. */
+template <int WAVES, int NB, bool CAUSAL, bool MASK>
+__global__ void __launch_bounds__(64 * WAVES, 2)
+k_fa_fwd_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ q,
+               const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
+               int seq_q, int seq_k, int q_tiles, int total_work, int work_per_xcd,
+               int kv_group, float scale_log2, const int *__restrict__ key_mask, QNorm qnorm) {
+    extern __shared__ __align__(16) uint16_t lds[];     /* 2 GROUP stages of [K tile | V tile] */
+    constexpr int WQ = 16 * NB;                          /* queries per wave */
+    constexpr int BM = WQ * WAVES;
+    /* Key tiles between two barriers. Two for the 8-wave shape (one workgroup per CU, so the LDS
+     * has room for four stages): the waves of a workgroup then only meet every other tile, and
+     * the faster ones do not stand at a barrier while the slower ones finish every single tile. */
+    constexpr int GROUP = WAVES * NB >= 12 ? 2 : 1;
+
+    /* XCD-aware numbering: hardware deals workgroups round-robin to the 8
+     * XCDs, so id%8 is the XCD; give each XCD a contiguous slice of the
+     * head-major work list. */
+    const int work = (blockIdx.x % XCDS) * work_per_xcd + blockIdx.x / XCDS;
+    if (work >= total_work) return;
+    const int head = work / q_tiles;
+    int qt = work - head * q_tiles;
+    if (CAUSAL) qt = q_tiles - 1 - qt;             /* longest rows first */
+    const int q0 = qt * BM;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    fa_walk_hd128<WAVES, NB, GROUP, CAUSAL, MASK>(lds, out, ldo, q, k, v, ldi, seq_q, seq_k, head, head / kv_group, q0, BM,
+                                                  q0 + wave * WQ, scale_log2, key_mask, qnorm);
+}
+
+/* The last, partly filled round of the kernel above leaves CUs idle: 432 workgroups on 256 CUs run as 256 + 176.
+ * Here a call is cut into workgroups of two sizes instead, so that its last round uses every CU for a shorter
+ * time: per head `full_tiles` workgroups of 256 queries as above, and behind them `tail_tiles` workgroups of 192
+ * queries, in which waves 0-3 carry 32 queries and waves 4-7 carry 16 (every SIMD then has three blocks of 16
+ * queries instead of four). The 256-query workgroups of all heads are numbered first, so they are dispatched
+ * first; each XCD takes its slice of both lists. */
+template <bool CAUSAL, bool MASK>
+__global__ void __launch_bounds__(512, 2)
+k_fa_fwd_hd128_two_sizes(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ q,
+                         const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
+                         int seq_q, int seq_k, int full_tiles, int total_full, int full_per_xcd,
+                         int tail_tiles, int total_tail, int tail_per_xcd,
+                         int kv_group, float scale_log2, const int *__restrict__ key_mask, QNorm qnorm) {
+    extern __shared__ __align__(16) uint16_t lds[];     /* four stages of [K tile | V tile] */
+    const int xcd = blockIdx.x % XCDS, slot = blockIdx.x / XCDS;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int head, q0, bm, wq0;
+    bool two_blocks;
+    if (slot < full_per_xcd) {
+        const int work = xcd * full_per_xcd + slot;
+        if (work >= total_full) return;
+        head = work / full_tiles;
+        q0 = (work - head * full_tiles) * 256; bm = 256;
+        wq0 = q0 + 32 * wave; two_blocks = true;
+    } else {
+        const int work = xcd * tail_per_xcd + slot - full_per_xcd;
+        if (work >= total_tail) return;
+        head = work / tail_tiles;
+        q0 = full_tiles * 256 + (work - head * tail_tiles) * 192; bm = 192;
+        two_blocks = wave < 4;
+        wq0 = two_blocks ? q0 + 32 * wave : q0 + 128 + 16 * (wave - 4);
+    }
+    if (two_blocks)
+        fa_walk_hd128<8, 2, 2, CAUSAL, MASK>(lds, out, ldo, q, k, v, ldi, seq_q, seq_k, head, head / kv_group, q0, bm, wq0,
+                                             scale_log2, key_mask, qnorm);
+    else
+        fa_walk_hd128<8, 1, 2, CAUSAL, MASK>(lds, out, ldo, q, k, v, ldi, seq_q, seq_k, head, head / kv_group, q0, bm, wq0,
+                                             scale_log2, key_mask, qnorm);
 }
 
 /* ---- short sequences ----------------------------------------------------------------------------
@@ -1008,6 +1066,29 @@ int launch(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint
     return (int)hipGetLastError();
 }
 
+template <bool C, bool M>
+int launch_two_sizes(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
+                     const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads,
+                     float scale, const int *key_mask, const QNorm &qn, int full_tiles) {
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd128_two_sizes<C, M>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
+        if (e != hipSuccess) return (int)e;
+        configured = true;
+    }
+    const int rest = seq_q - 256 * full_tiles;
+    const int tail_tiles = rest > 0 ? (rest + 191) / 192 : 0;
+    const int total_full = full_tiles * heads, total_tail = tail_tiles * heads;
+    const int full_per_xcd = (total_full + XCDS - 1) / XCDS, tail_per_xcd = (total_tail + XCDS - 1) / XCDS;
+    const size_t lds_bytes = stage_bytes<8, 2>() + (M ? 8 * (size_t)((seq_k + BN - 1) / BN) : 0);
+    if (lds_bytes > LDS_MAX) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL((k_fa_fwd_hd128_two_sizes<C, M>), dim3((full_per_xcd + tail_per_xcd) * XCDS), dim3(512), lds_bytes, st,
+                       out, ldo, q, k, v, ldi, seq_q, seq_k, full_tiles, total_full, full_per_xcd, tail_tiles, total_tail,
+                       tail_per_xcd, heads / kv_heads, scale * 1.4426950408889634f, key_mask, qn);
+    return (int)hipGetLastError();
+}
+
 template <int W, int NB = 2>
 int launch_w(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
              const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads, float scale,
@@ -1049,6 +1130,32 @@ int launch_short_cm(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, c
 }
 
 }  // namespace
+
+/* When the last of `n_full` workgroups of cost 100 followed by `n_tail` of cost `tail_cost` ends, if they are dealt in
+ * that order to the 256 CUs, each to the CU that is free first (which is what the dispatcher does with one
+ * workgroup per CU). The CUs are kept as groups that become free together; a step deals to one whole group. */
+static long makespan(long n_full, long n_tail, long tail_cost) {
+    struct Group { long free_at, cus; } g[3] = {{0, CUS}};            /* a group splits twice at most */
+    int ng = 1;
+    long left[2] = {n_full, n_tail}, end = 0;
+    const long cost[2] = {100, tail_cost};
+    for (int kind = 0; kind < 2; kind++)
+        while (left[kind] > 0) {
+            int first = 0;
+            for (int i = 1; i < ng; i++)
+                if (g[i].free_at < g[first].free_at) first = i;
+            const long take = g[first].cus < left[kind] ? g[first].cus : left[kind];
+            const long done = g[first].free_at + cost[kind];
+            left[kind] -= take;
+            if (done > end) end = done;
+            if (take == g[first].cus) g[first].free_at = done;          /* the whole group moves on */
+            else {                                                      /* the last of their kind: the group splits */
+                g[first].cus -= take;
+                g[ng].free_at = done; g[ng].cus = take; ng++;
+            }
+        }
+    return end;
+}
 
 static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
                             const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads, float scale,
@@ -1098,6 +1205,29 @@ static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16
     const long cost8 = 100 * ((wg256 + CUS - 1) / CUS);
     const long rest4 = wg128 % (2 * CUS);
     const long cost4 = 113 * (wg128 / (2 * CUS)) + (rest4 == 0 ? 0 : rest4 <= CUS ? 72 : 113);
+    if (!causal && cost8 <= cost4) {
+        /* 256-query workgroups whose last round is partly filled: cut the call into two sizes if that shortens it
+         * (k_fa_fwd_hd128_two_sizes). A round of 192-query workgroups costs 0.77 of a full one on the bench data
+         * and 0.83-0.86 on unnormalised N(0,1) rows (0.82 here); a last round of 256-query workgroups on at most 176
+         * CUs costs 0.88 (higher clock). 24 heads x 4608: 224 us against 237 (10 workgroups of 256 queries per head,
+         * then 11 of 192); 24 x 8704: 867 against 936; 24 x 16896: 3075 against 3220; what the model rejects is
+         * slower when forced (30 heads x 4352 as 10 + 10: 299 us against 239; 24 x 12800 as 40 + 14: 1843 against
+         * 1675) or gains 1 % (as 42 + 11: 1658). */
+        const long rem = wg256 % CUS;
+        const long cost_one_size = 100 * (wg256 / CUS) + (rem == 0 ? 0 : rem <= 176 ? 88 : 100);
+        long best_cost = cost_one_size * 985 / 1000;
+        int best_full = -1;
+        if (rem != 0)
+            for (int f = seq_q / 256; f >= 0; f--) {
+                const long tails = (seq_q - 256 * f + 191) / 192;
+                const long c = makespan((long)f * heads, tails * heads, 82);
+                if (c < best_cost) { best_cost = c; best_full = f; }
+            }
+        if (best_full >= 0) {
+            if (key_mask) return launch_two_sizes<false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn, best_full);
+            return launch_two_sizes<false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn, best_full);
+        }
+    }
     if (cost8 <= cost4)
         return launch_w<8>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
     return launch_w<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);

@@ -122,11 +122,13 @@ def test_c2_full_size_sampled_rows_and_properties(dev, orc):
     (1300, 16, 16, False, False), (1300, 16, 8, True, True),         # eight
     (2100, 24, 8, False, True), (2100, 24, 24, True, False),         # 32 queries per wave: 128- or 256-query workgroups
     (4200, 8, 8, False, False), (1500, 24, 24, False, True),
+    (4608, 24, 24, False, True), (8704, 24, 8, False, False),        # workgroups of two sizes: 256 queries, then 192
 ])
 def test_every_workgroup_width(dev, orc, seq, heads, kv, causal, masked):
     """The launcher picks the workgroup from the problem size: 1, 2, 4 or 8 waves of 16 queries for up to 2048 such
-    waves, 4 or 8 waves of 32 queries beyond (or, for few workgroups and many key tiles, the kernel that splits the
-    keys over the waves); each shape is its own instantiation of the kernel (pieces of a key tile per wave, LDS stages).
+    waves, 4 or 8 waves of 32 queries beyond, the last ones of a head with 32 and 16 queries per wave when that evens
+    out the last round (or, for few workgroups and many key tiles, the kernel that splits the keys over the waves);
+    each shape is its own instantiation of the kernel (pieces of a key tile per wave, LDS stages).
     Sampled rows against the oracle, including the rows around every workgroup boundary."""
     rng = np.random.default_rng(seq + heads)
     ldi = (heads + 2 * kv) * 128
