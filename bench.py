@@ -24,7 +24,10 @@ fused Q+K, rows in the Infinity Cache) and the kernel-only durations on file.
 (mean / median / min / single launch) with its fraction of the matrix peak,
 the norm+rope calls with their fraction of the HBM peak, the whole step
 (two norm+rope calls and attention) issued call by call and replayed from a
-HIP graph of 16 steps, and the seconds of the CPU port on this host's cores; `other_ops` the other device operators
+HIP graph of 16 steps, for a configuration with a key mask the number of valid
+keys drawn from the seed and the same launch with every key valid (the kernel
+stops at the last key tile that holds a valid key), and the seconds of the CPU
+port on this host's cores; `other_ops` the other device operators
 at this configuration's shapes, among them the q | k | v projection with
 and without the normalisation in its epilogue; `rope_tables` the time to
 build one forward pass's rotary tables (host builder + upload, and straight
@@ -798,6 +801,17 @@ def main():
                      "norm_rope_qk_frac_of_hbm_peak": round(nb / qk_ms / 1e6 / PEAK_HBM_GBPS, 4)}
             eager_us, graph_us = step_times(hip, stream, lib, r.step)
             entry.update(step_us=round(eager_us, 2), step_us_in_hip_graph=round(graph_us, 2))
+            if c["key_mask"] is not None:
+                # the kernel stops at the last key tile that holds a valid key, so the time depends on the mask drawn
+                # from the seed: the same launch with every key valid is timed beside it
+                drawn, every = r.mask, dev.to_device(np.ones(c["seq"], np.int32))
+                r.mask = every
+                settle(lib, r.attention, args.settle_ms / 10)
+                entry.update(valid_keys=int((c["key_mask"] != 0).sum()), attention_ms_with_every_key_valid=round(
+                    float(np.mean(per_launch_times(hip, stream, r.attention, n))), 4))
+                r.mask = drawn
+                lib.iris_dev_sync()
+                lib.iris_dev_free(every)
             dev.check()
             r.free()
             if not args.no_cpu:
