@@ -1131,11 +1131,16 @@ int launch_short_cm(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, c
 
 }  // namespace
 
-/* When the last of `n_full` workgroups of cost 100 followed by `n_tail` of cost `tail_cost` ends, if they are dealt in
- * that order to the 256 CUs, each to the CU that is free first (which is what the dispatcher does with one
- * workgroup per CU). The CUs are kept as groups that become free together; a step deals to one whole group. */
-static long makespan(long n_full, long n_tail, long tail_cost) {
-    struct Group { long free_at, cus; } g[3] = {{0, CUS}};            /* a group splits twice at most */
+/* How the hardware deals the workgroups of a grid, as far as timing shows it: workgroup i goes to XCD i % 8, the
+ * k-th workgroup of an XCD to its shader engine k % 4, whatever is free elsewhere, and a shader engine hands its
+ * workgroups in order to whichever of its 8 CUs is free first. (Measured on the two-size kernel for every number of
+ * 256-query workgroups per head on nine shapes: this rule reproduces every step of the curves to 2-3 %, a rule
+ * that pools the 256 CUs does not.) So a grid is as fast as its most loaded shader engine.
+ *
+ * When the last of `n_full` workgroups of cost 100 followed by `n_tail` of cost `tail_cost` ends on the `cus` CUs of a
+ * shader engine. The CUs are kept as groups that become free together; a step deals to one whole group. */
+static long makespan(long n_full, long n_tail, long tail_cost, long cus) {
+    struct Group { long free_at, cus; } g[3] = {{0, cus}};            /* a group splits twice at most */
     int ng = 1;
     long left[2] = {n_full, n_tail}, end = 0;
     const long cost[2] = {100, tail_cost};
@@ -1155,6 +1160,19 @@ static long makespan(long n_full, long n_tail, long tail_cost) {
             }
         }
     return end;
+}
+
+/* The two-size grid (k_fa_fwd_hd128_two_sizes) on its most loaded XCD, the first: workgroups k = 0 .. fx - 1 of the
+ * XCD are the 256-query ones, k = fx .. fx + tx - 1 the 192-query ones, and k % 4 is the shader engine. */
+static long two_sizes_cost(long n_full, long n_tail) {
+    const long fx = (n_full + XCDS - 1) / XCDS, tx = (n_tail + XCDS - 1) / XCDS;
+    long worst = 0;
+    for (long s = 0; s < 4; s++) {
+        const long full = fx > s ? (fx - s + 3) / 4 : 0, both = fx + tx > s ? (fx + tx - s + 3) / 4 : 0;
+        const long c = makespan(full, both - full, 78, CUS / XCDS / 4);
+        if (c > worst) worst = c;
+    }
+    return worst;
 }
 
 static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
@@ -1179,9 +1197,9 @@ static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16
      * Beyond that, 32 queries per wave, and the choice is between 256 queries (8 waves, one workgroup fills a CU,
      * half the K/V traffic from L2 per query) and 128 queries (4 waves, two workgroups per CU), by the cost of
      * their rounds over the 256 CUs, in units of one full round of 256-query workgroups: such a round costs 1
-     * however few CUs it uses; a round of 128-query workgroups costs 1.13 when some CU gets two of them and 0.72
-     * when none does (one wave per SIMD runs faster than two, not twice as fast). Constants measured on 24 heads,
-     * 256 .. 12800 tokens, clocks settled. */
+     * however few CUs it uses; a round of 128-query workgroups costs 1.1 when some CU gets two of them and 0.6
+     * when none does (one wave per SIMD runs faster than two, not twice as fast). Constants measured on 16 to 48
+     * heads, 256 .. 12800 tokens, clocks settled. */
     const long waves16 = (long)((seq_q + 15) / 16) * heads;
     if (waves16 <= 8 * CUS) {
         const int w = waves16 <= CUS ? 1 : waves16 <= 640 ? 2 : waves16 <= 4 * CUS ? 4 : 8;
@@ -1204,25 +1222,23 @@ static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16
     const long wg256 = (long)((seq_q + 255) / 256) * heads, wg128 = (long)((seq_q + 127) / 128) * heads;
     const long cost8 = 100 * ((wg256 + CUS - 1) / CUS);
     const long rest4 = wg128 % (2 * CUS);
-    const long cost4 = 113 * (wg128 / (2 * CUS)) + (rest4 == 0 ? 0 : rest4 <= CUS ? 72 : 113);
-    if (!causal && cost8 <= cost4) {
-        /* 256-query workgroups whose last round is partly filled: cut the call into two sizes if that shortens it
-         * (k_fa_fwd_hd128_two_sizes). A round of 192-query workgroups costs 0.77 of a full one on the bench data
-         * and 0.83-0.86 on unnormalised N(0,1) rows (0.82 here); a last round of 256-query workgroups on at most 176
-         * CUs costs 0.88 (higher clock). 24 heads x 4608: 224 us against 237 (10 workgroups of 256 queries per head,
-         * then 11 of 192); 24 x 8704: 867 against 936; 24 x 16896: 3075 against 3220; what the model rejects is
-         * slower when forced (30 heads x 4352 as 10 + 10: 299 us against 239; 24 x 12800 as 40 + 14: 1843 against
-         * 1675) or gains 1 % (as 42 + 11: 1658). */
-        const long rem = wg256 % CUS;
-        const long cost_one_size = 100 * (wg256 / CUS) + (rem == 0 ? 0 : rem <= 176 ? 88 : 100);
-        long best_cost = cost_one_size * 985 / 1000;
+    const long cost4 = 110 * (wg128 / (2 * CUS)) + (rest4 == 0 ? 0 : rest4 <= CUS ? 60 : 110);
+    if (!causal && cost8 <= 1000) {
+        /* Whatever the one-size kernels leave idle in their last round, two sizes may fill (k_fa_fwd_hd128_two_sizes):
+         * every number f of 256-query workgroups per head is priced with the dispatch rule above, a 192-query
+         * workgroup at 0.78 of a 256-query one, and the best f is taken if it beats both one-size kernels by 3 %.
+         * 24 heads x 4608: 224 us (f = 10, then 11 of 192 queries) against 237 and 262 for the 8- and 4-wave
+         * kernels; x 3072: 131 (f <= 6) against 160 / 143; x 5632: 351 (f = 4) against 428 / 404; 16 x 4608: 188
+         * against 231 / 206; 24 x 12800 gains 1 % and 30 x 4352 nothing (two full rounds). Over 77 shapes (16 to 48
+         * heads, 2304 to 8704 tokens) the choice made here is within 2 % of the best of the 4-wave kernel, the 8-wave
+         * kernel and every f on 70 of them and within 5 % on all. Beyond ten rounds the last one no longer matters. */
+        long best_cost = (cost8 <= cost4 ? cost8 : cost4) * 97 / 100;
         int best_full = -1;
-        if (rem != 0)
-            for (int f = seq_q / 256; f >= 0; f--) {
-                const long tails = (seq_q - 256 * f + 191) / 192;
-                const long c = makespan((long)f * heads, tails * heads, 82);
-                if (c < best_cost) { best_cost = c; best_full = f; }
-            }
+        for (int f = seq_q / 256; f >= 0; f--) {
+            const long tails = (seq_q - 256 * f + 191) / 192;
+            const long c = two_sizes_cost((long)f * heads, tails * heads);
+            if (c < best_cost) { best_cost = c; best_full = f; }
+        }
         if (best_full >= 0) {
             if (key_mask) return launch_two_sizes<false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn, best_full);
             return launch_two_sizes<false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn, best_full);
