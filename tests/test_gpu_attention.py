@@ -291,6 +291,20 @@ def test_ragged_shapes(dev, orc, fa, seq_q, seq_k, causal):
     assert_close(O.bf16_to_f32(out[:seq_q]), want, f"{seq_q}x{seq_k} causal={causal}")
 
 
+@pytest.mark.parametrize("seq_q,seq_k,heads,kv", [(3000, 5000, 24, 24), (5000, 3000, 16, 4), (2817, 70, 24, 8)])
+def test_large_calls_with_different_query_and_key_counts(dev, orc, fa, seq_q, seq_k, heads, kv):
+    """The workgroups are cut by the number of queries alone (one size, or 256 queries then 192); the keys only set the
+    length of the walk. Sampled query rows against the oracle, with the last rows of both workgroup sizes among them."""
+    buf, ldi = random_case(seq_q + seq_k, seq_q, seq_k, heads, kv)
+    qd, kd = heads * 128, kv * 128
+    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, 128, 0.0884, False)
+    assert kernel == fa
+    rows = np.unique(np.r_[sample_rows(seq_q, n=30, seed=seq_k), [255, 256, 447, 448, seq_q - 193, seq_q - 192, seq_q - 65, seq_q - 64]])
+    rows = rows[(rows >= 0) & (rows < seq_q)].astype(np.int32)
+    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, 128, 0.0884, False, None, rows=rows)
+    assert_close(O.bf16_to_f32(out[:seq_q])[rows], want, f"{seq_q} queries x {seq_k} keys")
+
+
 def test_random_key_masks_and_empty_rows(dev, orc, fa):
     heads, seq = 3, 300
     buf, ldi = random_case(5, seq, seq, heads, heads)
