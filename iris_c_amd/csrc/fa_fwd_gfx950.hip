@@ -369,17 +369,7 @@ fa_walk_hd128(uint16_t *__restrict__ lds, uint16_t *__restrict__ out, int ldo, c
 #pragma unroll
     for (int par = 0; par < 2; par++)
         lane_off[par] = (uint32_t)((lane >> 4) * ldi + 8 * ((lane & 15) ^ swz(4 * par + (lane >> 4)))) * 2u;
-    /* The key mask as one 64-bit word per key tile, kept in LDS behind the stages: built once here,
-     * so that the loop has no global load of its own (a load there would be waited for with
-     * vmcnt(0), i.e. together with the newest tile requests). Keys past seq_k count as masked. */
     unsigned long long *mask_words = reinterpret_cast<unsigned long long *>(lds + NSTAGE * STAGE);
-    if (MASK) {
-        for (int t = wave; t < ntiles; t += WAVES) {
-            const int key = t * BN + lane;
-            const unsigned long long word = __ballot(key < seq_k && key_mask[min(key, seq_k - 1)] != 0);
-            if (lane == 0) mask_words[t] = word;
-        }
-    }
 
     const int last_k0 = (ntiles - 1) * BN;
     auto request = [&](int tile_index, int stage) {      /* tile indices past the end repeat the last tile */
@@ -417,6 +407,28 @@ fa_walk_hd128(uint16_t *__restrict__ lds, uint16_t *__restrict__ out, int ldo, c
     if (qnorm.w) {                                   /* wave-uniform */
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) norm_rope_q_fragment(qb[nb], qnorm, min(qrow0 + 16 * nb, seq_q - 1), lg);
+    }
+
+    /* The key mask as one 64-bit word per key tile, kept in LDS behind the stages: built once here,
+     * so that the loop has no global load of its own (a load there would be waited for with
+     * vmcnt(0), i.e. together with the newest tile requests). Keys past seq_k count as masked. Behind the
+     * first tile requests and the Q loads, so that its round trips overlap theirs, and several tiles per wave
+     * at a time, so that 64 tiles cost a workgroup of 8 waves one round trip and not eight. */
+    if (MASK) {
+        constexpr int U = GROUP == 2 ? 8 : 2;               /* the small shapes walk few tiles: two per wave at a time */
+        for (int t0 = wave; t0 < ntiles; t0 += U * WAVES) {
+            int flag[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int key = (t0 + u * WAVES) * BN + lane;
+                flag[u] = key < seq_k ? key_mask[key] : 0;         /* tiles past the last one: key >= seq_k */
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const unsigned long long word = __ballot(flag[u] != 0);
+                if (lane == 0 && t0 + u * WAVES < ntiles) mask_words[t0 + u * WAVES] = word;
+            }
+        }
     }
 
     /* The tile requests are invisible to the compiler's own wait-count bookkeeping, so every load it
