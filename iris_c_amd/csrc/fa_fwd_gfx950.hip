@@ -1187,9 +1187,11 @@ static long two_sizes_cost(long n_full, long n_tail) {
     return worst;
 }
 
-static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
-                            const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads, float scale,
-                            int causal, const int *key_mask, const QNorm &qn) {
+/* Which kernel a call takes: kind 0 = k_fa_fwd_hd128<waves, nb>, 1 = k_fa_fwd_hd128_two_sizes with `full` workgroups
+ * of 256 queries per head, 2 = k_fa_short_hd128<split>. Host arithmetic only. */
+struct FaPlan { int kind, waves, nb, split, full; };
+
+static FaPlan plan_hd128(int seq_q, int seq_k, int heads, int causal) {
     /* Three regimes, by the number of waves of 16 queries the problem makes (heads x ceil(seq_q / 16)).
      *
      * Up to 2048 of them (one wave per SIMD and CU slot, or fewer): a workgroup walks its key tiles one after the
@@ -1202,8 +1204,8 @@ static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16
      * workgroup, 0.92 with four, 1.08 with eight.
      * When the (head, 32-query block) pairs are at most one per CU and the sequence has many key tiles, splitting
      * the keys over the waves of a workgroup (k_fa_short_hd128) is shorter still: 1.45 us per turn of
-     * ceil(tiles / S) plus 1.5 for the merge. 1 head x 512 tokens 9.0 us against 9.8; 8 heads x 1024 14.9 against
-     * 16.9; 4 heads x 2000 + mask 25.4 against 32.5. (With more than one workgroup per CU its private tiles cost
+     * ceil(tiles / 4) (S = 4 waves) plus 1.5 for the merge, which pays from seven tiles on. 1 head x 512 tokens
+     * 9.0 us against 9.8; 8 heads x 1024 14.9 against 16.9; 4 heads x 2000 + mask 25.4 against 32.5. (With more than one workgroup per CU its private tiles cost
      * what the shorter chain saves: 32 heads x 512 tokens, 512 workgroups, 16.4 us.)
      *
      * Beyond that, 32 queries per wave, and the choice is between 256 queries (8 waves, one workgroup fills a CU,
@@ -1219,17 +1221,8 @@ static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16
         const long keys = causal ? (seq_k < 32 * q_tiles32 ? seq_k : 32 * q_tiles32) : seq_k;
         const long tiles = (keys + BN - 1) / BN;
         const long cost_chain = tiles * (w <= 2 ? 65 : w == 4 ? 92 : 108);           /* 0.01 us */
-        if (tiles >= 2 && q_tiles32 * heads <= CUS) {
-            const int s = tiles >= 6 ? 4 : 2;
-            if (((tiles + s - 1) / s) * 145 + 150 < cost_chain) {
-                if (s == 4) return launch_short_cm<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
-                return launch_short_cm<2>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
-            }
-        }
-        if (w == 1) return launch_w<1, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
-        if (w == 2) return launch_w<2, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
-        if (w == 4) return launch_w<4, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
-        return launch_w<8, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+        if (q_tiles32 * heads <= CUS && ((tiles + 3) / 4) * 145 + 150 < cost_chain) return {2, 4, 2, 4, 0};   /* from 7 tiles on */
+        return {0, w, 1, 0, 0};
     }
     const long wg256 = (long)((seq_q + 255) / 256) * heads, wg128 = (long)((seq_q + 127) / 128) * heads;
     const long cost8 = 100 * ((wg256 + CUS - 1) / CUS);
@@ -1251,14 +1244,37 @@ static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16
             const long c = two_sizes_cost((long)f * heads, tails * heads);
             if (c < best_cost) { best_cost = c; best_full = f; }
         }
-        if (best_full >= 0) {
-            if (key_mask) return launch_two_sizes<false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn, best_full);
-            return launch_two_sizes<false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn, best_full);
-        }
+        if (best_full >= 0) return {1, 8, 2, 0, best_full};
     }
-    if (cost8 <= cost4)
-        return launch_w<8>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+    return {0, cost8 <= cost4 ? 8 : 4, 2, 0, 0};
+}
+
+static int launch_any_width(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
+                            const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads, float scale,
+                            int causal, const int *key_mask, const QNorm &qn) {
+    const FaPlan p = plan_hd128(seq_q, seq_k, heads, causal);
+    if (p.kind == 2) return launch_short_cm<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+    if (p.kind == 1) {
+        if (key_mask) return launch_two_sizes<false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn, p.full);
+        return launch_two_sizes<false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, key_mask, qn, p.full);
+    }
+    if (p.nb == 1) {
+        if (p.waves == 1) return launch_w<1, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+        if (p.waves == 2) return launch_w<2, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+        if (p.waves == 4) return launch_w<4, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+        return launch_w<8, 1>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+    }
+    if (p.waves == 8) return launch_w<8>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
     return launch_w<4>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, qn);
+}
+
+/* The launcher's choice for a head_dim-128 call, without launching anything (no GPU needed): plan[0] = kind (0 one
+ * size, 1 two sizes, 2 keys split over the waves), plan[1] = waves per workgroup, plan[2] = blocks of 16 queries per
+ * wave, plan[3] = 256-query workgroups per head of the two-size grid, plan[4] = its 192-query workgroups per head. */
+extern "C" void iris_hip_fa_hd128_plan(int seq_q, int seq_k, int heads, int causal, int *plan) {
+    const FaPlan p = plan_hd128(seq_q, seq_k, heads, causal);
+    plan[0] = p.kind; plan[1] = p.waves; plan[2] = p.nb; plan[3] = p.full;
+    plan[4] = p.kind == 1 ? (seq_q - 256 * p.full + 191) / 192 : 0;
 }
 
 extern "C" int iris_hip_fa_hd128(void *stream, uint16_t *out, int ldo, const uint16_t *q,

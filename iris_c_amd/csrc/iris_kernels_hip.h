@@ -49,6 +49,12 @@ int iris_hip_fa_hd128_qnorm(void *stream, uint16_t *out, int ldo, const uint16_t
                             const float *w, const float *rope_cos, const float *rope_sin, float eps,
                             int split_half);
 
+/* What iris_hip_fa_hd128 would launch for these sizes, host arithmetic only (no GPU needed): plan[0] = 0 one size
+ * of workgroup, 1 two sizes (256 queries, then 192), 2 keys split over the waves of a workgroup; plan[1] = waves per
+ * workgroup; plan[2] = blocks of 16 queries per wave; plan[3], plan[4] = 256- and 192-query workgroups per head of
+ * the two-size grid. */
+void iris_hip_fa_hd128_plan(int seq_q, int seq_k, int heads, int causal, int *plan);
+
 /* head_dim 256 or 512 (the VAE's single 512-wide head): the head dim is cut into slices of
  * 128 that a group of waves shares; same argument conditions as iris_hip_fa_hd128. */
 int iris_hip_fa_sliced(void *stream, uint16_t *out, int ldo, const uint16_t *q,
