@@ -234,8 +234,8 @@ def test_c3_full_size_masked_equals_compacted(dev, orc, fa):
 
 # ------------------------------------------------------------------ edge cases
 @pytest.mark.parametrize("seq_q,seq_k,heads,kv,causal,masked", [
-    (77, 333, 8, 2, False, True),          # six key tiles over four waves: two waves take two tiles
-    (40, 130, 3, 3, False, False),         # three tiles over two waves
+    (77, 400, 8, 2, False, True),          # seven key tiles over four waves: three waves take two tiles
+    (40, 130, 3, 3, False, False),         # three tiles: below the length where the split pays, one wave walks them
     (500, 500, 4, 2, True, True),          # causal: the waves of the first query blocks have no tile at all
     (1000, 1000, 2, 2, True, True),        # four tiles per wave: the masks of the later ones are read in the loop
     (33, 3000, 1, 1, False, True),         # twelve turns per wave, ragged last tile
