@@ -11,9 +11,11 @@
  * the 16x16 accumulator a lane then holds four consecutive n of one output row m,
  * a single 16-byte (f32) or 8-byte (bf16) store.
  *
- * Two kernels. Shapes with M, N >= 256 and K a multiple of 64 (every linear layer of the models at
- * their sequence lengths) take k_gemm_dma: 256 x 256 tiles, 8 waves, tiles loaded straight into
- * LDS, described where it is defined. Everything else with K a multiple of 8 takes k_gemm_bf16:
+ * Three kernels. Whole 256 x 256 tiles with K a multiple of 128 (every linear layer of the models at
+ * their sequence lengths) take k_gemm_w4: four waves of 128 x 128 outputs, one per SIMD, tiles staged
+ * through registers. Other shapes with M, N >= 256 and K a multiple of 64, and the convolutions, take
+ * k_gemm_dma: the same tiles on 8 waves, loaded straight into LDS. Both are described where they are
+ * defined and give the same bits. Everything else with K a multiple of 8 takes k_gemm_bf16:
  * Workgroup = WM x WN waves (2 x 2 in use), tile 128 (m) x 128 (n), K in steps of 64; a wave owns
  * 64 x 64 = 4 x 4 accumulator blocks and reads 8 operands from LDS per 16 MFMAs. One
  * LDS stage of [W tile | x tile], rows padded to 160 B so that the 16 lanes the LDS
@@ -486,6 +488,278 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
         }
     }
 }
+/* ---- the same 256 x 256 x 64 tiles on FOUR waves, one per SIMD with the whole register file ----
+ *
+ * For whole tiles (M, N multiples of 256, K a multiple of 128). Each wave owns 128 x 128 outputs = 8 x 8
+ * accumulator blocks, 256 registers that live in AGPRs (the products are asm statements, so that they stay there),
+ * so an operand read from the LDS feeds eight products: 32 reads per 128 MFMAs and k tile, two thirds of the LDS
+ * traffic of the 8-wave kernel. A wave that is alone on its SIMD has nobody to hide its other instructions behind:
+ * it issues in order, and what stands between two products must fit into the 12 cycles the matrix core still
+ * works on the first. Hence
+ *  - the tiles are staged through registers (a direct HBM -> LDS load blocks the issuing wave for about 100
+ *    cycles): 16 loads of 16 B per thread and k tile, two tiles ahead (two register sets), each written to the
+ *    LDS as two 8-byte halves (a 16-byte LDS write takes longer to issue than the gap: 1265 -> 1302 TFLOP/s);
+ *  - every gap between two products holds at most one memory instruction: odd gaps of steps 0 - 2 the copies
+ *    registers -> LDS of tile kt + 1 and the loads of tile kt + 3, even gaps the operand reads of the next step
+ *    (all of them bunched at the step boundaries: 1160 TFLOP/s; two and a load per fourth gap: 1230; one per gap:
+ *    1253);
+ *  - one barrier per k tile, behind the products of step 2.
+ * Same LDS layout as above (128 B rows, chunk c of row r in slot c ^ ((r >> 1) & 7)), two stages. Same bits as the
+ * 8-wave kernel (same products in the same order per accumulator). Timing-only ablations at 4608 x 3072 -> 27648,
+ * 1270 TFLOP/s as it stood then: without the barrier 1262 -> 1305 (+3.5 %), without the global loads 1451, without
+ * loads and LDS writes 1711 (what 128 MFMAs and 32 operand reads per k tile run at), with loads that always hit
+ * the same cached tile 1396. */
+template <typename OUT, bool QKN>
+__global__ void __launch_bounds__(256, 1)
+k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *__restrict__ W,
+          int M, int N, int K, int tiles_m, int total, int per_xcd, QkNorm qn) {
+    constexpr int TN = 256;
+    constexpr int STAGE = (TN + DT) * TK;                      /* elements: W tile then x tile */
+    constexpr int NC = 8;                                      /* chunks of W (and of x) per thread and k tile: rows srow + 32 c */
+    extern __shared__ __align__(16) uint16_t dlds[];          /* two stages (and room for the epilogue) */
+    const int work = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (work >= total) return;
+    constexpr int BAND = 4;
+    const int tiles_n = total / tiles_m;
+    const int band = work / (BAND * tiles_n), in_band = work - band * (BAND * tiles_n);
+    const int band_rows = min(tiles_m - band * BAND, BAND);
+    const int bm = band * BAND + in_band % band_rows, bn = in_band / band_rows;
+    const int m0 = bm * DT, n0 = bn * TN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+    const int wm = wave & 1, wn = wave >> 1;
+
+    /* staging: chunk tid % 8 of rows tid / 8 + 32 c; (row >> 1) & 7 is the same for all c. Whole tiles only
+     * (M and N multiples of 256), so no row is clamped and the 16 loads of a thread differ by uniform offsets. */
+    const int srow = tid >> 3, schunk = tid & 7;
+    const int st_off = srow * TK + 8 * (schunk ^ ((srow >> 1) & 7));
+    const char *wt = reinterpret_cast<const char *>(W + (size_t)n0 * K), *xt = reinterpret_cast<const char *>(x + (size_t)m0 * K);   /* uniform tile bases */
+    const uint32_t lane_b = (uint32_t)(srow * K + 8 * schunk) * 2u;            /* this thread's bytes into a tile row block: never changes */
+    uint32_t tile_b = 0;                                                        /* uniform: bytes of the k tile to fetch next */
+    const uint32_t cstride = 64u * (uint32_t)K;                                 /* 32 rows, in bytes */
+    const int nk = K / TK, nk_tiles = nk;
+    u32x4 wreg[2][NC], xreg[2][NC];                            /* two tiles on their way at any time */
+    int fetched = 0;                                           /* tiles requested so far; tile_b stays on the last tile at the end */
+    auto fetch_one = [&](int set, int c) {                     /* c < 8: chunk c of W, else chunk c - 8 of x */
+        if (c < NC) wreg[set][c] = *reinterpret_cast<const u32x4 *>(wt + (size_t)(tile_b + c * cstride) + lane_b);
+        else xreg[set][c - NC] = *reinterpret_cast<const u32x4 *>(xt + (size_t)(tile_b + (c - NC) * cstride) + lane_b);
+    };
+    auto fetched_tile = [&]() { fetched++; tile_b += fetched < nk_tiles ? 2u * TK : 0u; };
+    auto store_half = [&](int set, int stage, int c, int hi) {  /* 8 of the 16 bytes of chunk c */
+        uint16_t *w_dst = dlds + stage * STAGE + st_off + 4 * hi;
+        const u32x4 v = c < NC ? wreg[set][c] : xreg[set][c - NC];
+        uint16_t *dst = c < NC ? w_dst + 32 * c * TK : w_dst + TN * TK + 32 * (c - NC) * TK;
+        *reinterpret_cast<uint2 *>(dst) = hi ? make_uint2(v[2], v[3]) : make_uint2(v[0], v[1]);
+    };
+    auto store_one = [&](int set, int stage, int c) { store_half(set, stage, c, 0); store_half(set, stage, c, 1); };
+
+    f32x4 acc[8][8];                                           /* [a: 16 columns][b: 16 rows] */
+#pragma unroll
+    for (int a = 0; a < 8; a++)
+#pragma unroll
+        for (int b = 0; b < 8; b++) acc[a][b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    int a_rd[2], b_rd[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        const int slot = 8 * ((4 * ks + lg) ^ (li >> 1));
+        a_rd[ks] = (128 * wn + li) * TK + slot;
+        b_rd[ks] = TN * TK + (128 * wm + li) * TK + slot;
+    }
+
+    /* Four steps of 32 MFMAs per k tile: k-step ks = step / 2, x blocks 4 (step % 2) .. + 3. The operands of a step
+     * are requested from the LDS before the products of the step before it are issued, across the tile boundary
+     * too. One barrier per tile, behind the products of step 2: by then every wave has written its share of tile
+     * kt + 1 (step 0) and has read the last operands of tile kt (step 2), so after it the stage of tile kt + 1 is
+     * complete and the stage of tile kt is free for tile kt + 2. The products are asm statements with the
+     * accumulators in AGPRs; the copies registers -> LDS of tile kt + 1 and the loads of tile kt + 2 stand between
+     * the products of step 0, one of each behind every second product. */
+    u32x4 av[2][8], bv[2][4];
+    auto read_a_one = [&](const uint16_t *stage, int ks, int a) {
+        av[ks][a] = *reinterpret_cast<const u32x4 *>(&stage[a_rd[ks] + 16 * a * TK]);
+    };
+    auto read_b_one = [&](const uint16_t *stage, int step, int b) {
+        bv[step & 1][b] = *reinterpret_cast<const u32x4 *>(&stage[b_rd[step >> 1] + 16 * (4 * (step & 1) + b) * TK]);
+    };
+    auto products = [&](int step, auto &&between) {
+        const int ks = step >> 1, half = step & 1;
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+            for (int a = 0; a < 8; a++) {
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[a][4 * half + b]) : "v"(av[ks][a]), "v"(bv[step & 1][b]));
+                between(8 * b + a);
+            }
+    };
+
+#pragma unroll
+    for (int c = 0; c < 2 * NC; c++) fetch_one(0, c);          /* tile 0 */
+    fetched_tile();
+#pragma unroll
+    for (int c = 0; c < 2 * NC; c++) store_one(0, 0, c);
+#pragma unroll
+    for (int c = 0; c < 2 * NC; c++) fetch_one(1, c);          /* tiles 1 and 2 (or the last tile again) wait in the registers */
+    fetched_tile();
+#pragma unroll
+    for (int c = 0; c < 2 * NC; c++) fetch_one(0, c);
+    fetched_tile();
+    lds_barrier();
+#pragma unroll
+    for (int a = 0; a < 8; a++) read_a_one(dlds, 0, a);
+#pragma unroll
+    for (int b = 0; b < 4; b++) read_b_one(dlds, 0, b);
+
+    /* One k tile: `set` holds tile kt + 1 on entry and tile kt + 3 on exit. */
+    auto k_tile = [&](int kt, int set) {
+        const uint16_t *cur = dlds + (kt & 1) * STAGE, *nxt = dlds + ((kt + 1) & 1) * STAGE;
+        const int nstage = (kt + 1) & 1;
+        /* At most one memory instruction behind a product: the wave issues in order, and what it issues between
+         * two products has to fit into the 12 cycles the matrix core still works on the first. Odd slots of steps 0
+         * and 1: tile kt + 1 registers -> LDS (chunk c behind product 4 c + 1) and tile kt + 3 -> registers (behind
+         * 4 c + 3); even slots: the operands of the next step, in the order its products use them. */
+        auto slot = [&](int step, int i) {
+            if (step < 3 && (i & 1)) {                          /* odd slots of steps 0 - 2: 48 = 16 x (two halves, one load) */
+                const int j = 16 * step + (i >> 1), c = j / 3, part = j - 3 * c;
+                if (part < 2) store_half(set, nstage, c, part);
+                else fetch_one(set, c);
+            }
+            if ((i & 1) == 0) {
+                const int r = i >> 1;
+                if (step == 0 && r < 4) read_b_one(cur, 1, r);
+                if (step == 1) { if (r < 4) read_b_one(cur, 2, r); else if (r < 12) read_a_one(cur, 1, r - 4); }
+                if (step == 2 && r < 4) read_b_one(cur, 3, r);
+                if (step == 3) { if (r < 4) read_b_one(nxt, 0, r); else if (r < 12) read_a_one(nxt, 0, r - 4); }
+            }
+        };
+        products(0, [&](int i) { slot(0, i); });
+        products(1, [&](int i) { slot(1, i); });
+        products(2, [&](int i) { slot(2, i); });
+        fetched_tile();
+        lds_barrier();
+        products(3, [&](int i) { slot(3, i); });
+    };
+    for (int kt = 0; kt < nk; kt += 2) {                       /* nk is even */
+        k_tile(kt, 1);
+        k_tile(kt + 1, 0);
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");                /* the last products have left the matrix core before the accumulators are read */
+    lds_barrier();                                              /* the LDS is reused by the epilogue */
+
+    /* acc[a][b][r] = y[m0 + 128 wm + 16 b + li][n0 + 128 wn + 16 a + 4 lg + r] */
+    constexpr int PER16 = 16 / (int)sizeof(OUT);
+    const int mw = m0 + 128 * wm, nw = n0 + 128 * wn;
+    if constexpr (QKN) {
+        /* the whole 256 x 256 bf16 tile in the LDS (128 KB), then a 16-lane row per (token, head) vector: see k_gemm_dma */
+        static_assert(sizeof(OUT) == 2, "bf16 projection only");
+        if (n0 < qn.qk_cols) {
+#pragma unroll
+            for (int b = 0; b < 8; b++)
+#pragma unroll
+                for (int a = 0; a < 8; a++) {
+                    const int row = 128 * wm + 16 * b + li, chunk = 16 * wn + 2 * a + (lg >> 1);
+                    const int slot = (chunk & 16) | ((chunk ^ li) & 15);
+                    *reinterpret_cast<uint2 *>(&dlds[row * 256 + 8 * slot + 4 * (lg & 1)]) =
+                        make_uint2(pack_bf16(acc[a][b][0], acc[a][b][1]), pack_bf16(acc[a][b][2], acc[a][b][3]));
+                }
+            __syncthreads();
+            const int sub = tid & 15, head = (tid >> 4) & 1, row_in = tid >> 5;
+            const int n_head = n0 + 128 * head, n = n_head + 8 * sub;
+            const bool normed = n_head < qn.qk_cols;
+            float w8[8] = {};
+            if (normed) {
+                const float *wsel = (n_head < qn.q_cols ? qn.wq : qn.wk) + 8 * sub;
+                const float4 w0 = *reinterpret_cast<const float4 *>(wsel), w1 = *reinterpret_cast<const float4 *>(wsel + 4);
+                w8[0] = w0.x; w8[1] = w0.y; w8[2] = w0.z; w8[3] = w0.w; w8[4] = w1.x; w8[5] = w1.y; w8[6] = w1.z; w8[7] = w1.w;
+            }
+            const int tcol = qn.split_half ? 8 * (sub & 7) : 4 * sub;
+            const int chunk = 16 * head + sub;
+            /* whole tiles: no row or head of the tile lies outside y, so the passes are straight-line code and the
+             * table loads of eight of them are in flight together (the wave has its SIMD to itself: nothing else
+             * hides their latency) */
+#pragma unroll 8
+            for (int pass = 0; pass < DT / 8; pass++) {
+                const int row = 8 * pass + row_in, m = m0 + row;
+                u32x4 v = *reinterpret_cast<const u32x4 *>(&dlds[row * 256 + 8 * ((chunk & 16) | ((chunk ^ row) & 15))]);
+                if (normed) {
+                    const float *cr = qn.rope_cos + (size_t)m * 64 + tcol, *sr = qn.rope_sin + (size_t)m * 64 + tcol;
+                    float cv[8] = {}, sv[8] = {};
+                    const float4 c0 = *reinterpret_cast<const float4 *>(cr), s0 = *reinterpret_cast<const float4 *>(sr);
+                    cv[0] = c0.x; cv[1] = c0.y; cv[2] = c0.z; cv[3] = c0.w;
+                    sv[0] = s0.x; sv[1] = s0.y; sv[2] = s0.z; sv[3] = s0.w;
+                    if (qn.split_half) {
+                        const float4 c1 = *reinterpret_cast<const float4 *>(cr + 4), s1 = *reinterpret_cast<const float4 *>(sr + 4);
+                        cv[4] = c1.x; cv[5] = c1.y; cv[6] = c1.z; cv[7] = c1.w;
+                        sv[4] = s1.x; sv[5] = s1.y; sv[6] = s1.z; sv[7] = s1.w;
+                        v = nr_vector_hd128<true>(v, w8, cv, sv, qn.eps, sub);
+                    } else {
+                        v = nr_vector_hd128<false>(v, w8, cv, sv, qn.eps, sub);
+                    }
+                }
+                *reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(y) + (size_t)m * N + n) = v;
+            }
+            return;
+        }
+    }
+    const bool staged = N % PER16 == 0 && ((uintptr_t)y & 15) == 0;
+    if (staged) {
+        /* through the LDS (free after the loop's last barrier; 32 KB per wave, its own region, no workgroup barrier), so
+         * that the stores leave as 16 B per lane along the rows. LDS serves a wave's instructions in order. */
+        uint16_t *mine = dlds + wave * 16384;
+        if constexpr (sizeof(OUT) == 4) {
+            float *buf = reinterpret_cast<float *>(mine);       /* 64 rows x 128 f32 at a time, chunk c of row r in slot (c & 16) | ((c ^ r) & 15) */
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+#pragma unroll
+                for (int bb = 0; bb < 4; bb++)
+#pragma unroll
+                    for (int a = 0; a < 8; a++) {
+                        const int chunk = 4 * a + lg;
+                        *reinterpret_cast<f32x4 *>(&buf[(16 * bb + li) * 128 + 4 * ((chunk & 16) | ((chunk ^ li) & 15))]) = acc[a][4 * half + bb];
+                    }
+#pragma unroll
+                for (int it = 0; it < 32; it++) {
+                    const int row = 2 * it + (lane >> 5), c = lane & 31;
+                    f32x4 v = *reinterpret_cast<const f32x4 *>(&buf[row * 128 + 4 * ((c & 16) | ((c ^ row) & 15))]);
+                    const int m = mw + 64 * half + row, n = nw + 4 * c;
+                    if (m < M && n < N) {
+                        *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(y) + (size_t)m * N + n) = v;
+                    }
+                }
+            }
+        } else {
+            uint16_t *buf = mine;                               /* 128 rows x 128 bf16, chunk c of row r in slot c ^ (r % 16) */
+#pragma unroll
+            for (int b = 0; b < 8; b++)
+#pragma unroll
+                for (int a = 0; a < 8; a++) {
+                    const int chunk = 2 * a + (lg >> 1);
+                    *reinterpret_cast<uint2 *>(&buf[(16 * b + li) * 128 + 8 * (chunk ^ li) + 4 * (lg & 1)]) =
+                        make_uint2(pack_bf16(acc[a][b][0], acc[a][b][1]), pack_bf16(acc[a][b][2], acc[a][b][3]));
+                }
+#pragma unroll
+            for (int it = 0; it < 32; it++) {
+                const int row = 4 * it + (lane >> 4), c = lane & 15;
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(&buf[row * 128 + 8 * (c ^ (row & 15))]);
+                const int m = mw + row, n = nw + 8 * c;
+                if (m < M && n < N) *reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(y) + (size_t)m * N + n) = v;
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+        const int m = mw + 16 * b + li;
+        if (m >= M) continue;
+#pragma unroll
+        for (int a = 0; a < 8; a++) {
+            const int n = nw + 16 * a + 4 * lg;
+            if (n >= N) continue;
+            f32x4 v = acc[a][b];
+            store4(y + (size_t)m * N + n, v, N - n);
+        }
+    }
+}
+
 #pragma clang diagnostic pop
 
 constexpr int DMA_LDS_BYTES = 128 * 1024;        /* two stages of (256 + 256) x 128 B; also the 8 x 16 KB of the epilogue */
@@ -521,13 +795,33 @@ k_gemm_scalar(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_
     store4(y + i, v, 1);
 }
 
+template <typename OUT, bool QKN = false>
+int launch_gemm_w4(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, int N, int K, const QkNorm &qn = QkNorm{}) {
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_w4<OUT, QKN>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, DMA_LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        configured = true;
+    }
+    const int tiles_m = M / DT, tiles_n = N / 256, total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    hipLaunchKernelGGL((k_gemm_w4<OUT, QKN>), dim3((unsigned)per_xcd * 8), dim3(256), DMA_LDS_BYTES, st, y, x, W, M, N, K,
+                       tiles_m, total, per_xcd, qn);
+    return (int)hipGetLastError();
+}
+
+/* Whole 256 x 256 tiles and an even number of k tiles: what the four-wave kernel takes. */
+static bool whole_tiles(int M, int N, int K) { return M % DT == 0 && N % 256 == 0 && K % (2 * TK) == 0; }
+
 template <typename OUT>
 int gemm(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, int N, int K) {
     if (M <= 0 || N <= 0) return 0;
     const bool aligned16 = ((uintptr_t)x & 15) == 0 && ((uintptr_t)W & 15) == 0;
     if (K > 0 && K % TK == 0 && aligned16 && M >= DT && N >= DT && (size_t)K * 2 * 8 < ((size_t)1 << 31)) {
         const ConvGeom none = {};
-        const int e = launch_gemm_dma<OUT, 256, false>(st, y, x, W, M, N, K, none);
+        const int e = whole_tiles(M, N, K) ? launch_gemm_w4<OUT>(st, y, x, W, M, N, K)
+                                           : launch_gemm_dma<OUT, 256, false>(st, y, x, W, M, N, K, none);
         if (e) return e;
     } else if (K > 0 && K % 8 == 0 && aligned16) {
         /* 2 x 2 waves (128 x 128 tiles) measured best on the transformer shapes: 4 x 2 and 2 x 4 are
@@ -605,6 +899,7 @@ int iris_hip_linear_bf16_qknorm(void *stream, uint16_t *y, const uint16_t *x, co
         return -2;
     const ConvGeom none = {};
     const QkNorm qn = {wq, k_cols ? wk : wq, rope_cos, rope_sin, q_cols, q_cols + k_cols, eps, split_half};
+    if (whole_tiles(M, N, K)) return launch_gemm_w4<uint16_t, true>((hipStream_t)stream, y, x, W, M, N, K, qn);
     return launch_gemm_dma<uint16_t, 256, false, true>((hipStream_t)stream, y, x, W, M, N, K, none, qn);
 }
 

@@ -77,6 +77,9 @@ ONE_LAUNCH = [
     (512, 128, 3, 0, 128, 0),       # Q only, and a last tile of 128 columns
     (300, 192, 0, 1, 128, 1),       # K only
     (1000, 512, 5, 5, 0, 0),        # nothing after K; 1280 columns = five tiles
+    (512, 256, 2, 2, 256, 0),       # whole tiles and in % 128 == 0: the four-wave kernel's epilogue
+    (768, 384, 3, 1, 0, 1),         # the same, split halves, three query heads on one kv head
+    (256, 128, 1, 1, 256, 1),       # its smallest case: two k tiles, one tile with a Q and a K head, one without
 ]
 
 

@@ -45,7 +45,9 @@ def run(dev, fn, outs):
 @pytest.mark.parametrize("rows,k,out", [(1, 8, 1), (5, 64, 7), (128, 128, 128), (130, 200, 260), (333, 3072, 520), (64, 96, 64),
                                         # the 256 x 256 kernel (rows, out >= 256, k % 64 == 0): ragged edges, and an `out` that
                                         # rules out 16-byte stores (its epilogue then stores straight from the accumulators)
-                                        (300, 128, 258), (257, 64, 257), (512, 192, 256), (700, 256, 1000)])
+                                        (300, 128, 258), (257, 64, 257), (512, 192, 256), (700, 256, 1000),
+                                        # whole 256 x 256 tiles and k % 128 == 0: the four-wave kernel (two k tiles at least)
+                                        (256, 128, 256), (512, 256, 512), (768, 640, 1024)])
 @pytest.mark.parametrize("out_bf16", [False, True])
 @pytest.mark.parametrize("backend", ["library", "own"])
 def test_linear(dev, orc, rows, k, out, out_bf16, backend):
