@@ -11,9 +11,9 @@
  * the 16x16 accumulator a lane then holds four consecutive n of one output row m,
  * a single 16-byte (f32) or 8-byte (bf16) store.
  *
- * Three kernels. Whole 256 x 256 tiles with K a multiple of 128 (every linear layer of the models at
- * their sequence lengths) take k_gemm_w4: four waves of 128 x 128 outputs, one per SIMD, tiles staged
- * through registers. Other shapes with M, N >= 256 and K a multiple of 64, and the convolutions, take
+ * Three kernels. M, N >= 256 with K a multiple of 128 (every linear layer of the models at their
+ * sequence lengths) take k_gemm_w4: tiles of 256 rows x 256, 224 or 192 columns on four waves, one per
+ * SIMD, staged through registers. Other shapes with M, N >= 256 and K a multiple of 64, and the convolutions, take
  * k_gemm_dma: the same tiles on 8 waves, loaded straight into LDS. Both are described where they are
  * defined and give the same bits. Everything else with K a multiple of 8 takes k_gemm_bf16:
  * Workgroup = WM x WN waves (2 x 2 in use), tile 128 (m) x 128 (n), K in steps of 64; a wave owns
@@ -490,8 +490,8 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
 }
 /* ---- the same 256 x 256 x 64 tiles on FOUR waves, one per SIMD with the whole register file ----
  *
- * For whole tiles (M, N multiples of 256, K a multiple of 128). Each wave owns 128 x 128 outputs = 8 x 8
- * accumulator blocks, 256 registers that live in AGPRs (the products are asm statements, so that they stay there),
+ * For M, N >= 256 and K a multiple of 128. Each wave owns 128 rows x 16 NA columns = NA x 8 accumulator
+ * blocks, up to 256 registers that live in AGPRs (the products are asm statements, so that they stay there),
  * so an operand read from the LDS feeds eight products: 32 reads per 128 MFMAs and k tile, two thirds of the LDS
  * traffic of the 8-wave kernel. A wave that is alone on its SIMD has nobody to hide its other instructions behind:
  * it issues in order, and what stands between two products must fit into the 12 cycles the matrix core still
@@ -509,13 +509,15 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
  * 1270 TFLOP/s as it stood then: without the barrier 1262 -> 1305 (+3.5 %), without the global loads 1451, without
  * loads and LDS writes 1711 (what 128 MFMAs and 32 operand reads per k tile run at), with loads that always hit
  * the same cached tile 1396. */
-template <typename OUT, bool QKN>
+template <typename OUT, int NA, bool QKN>
 __global__ void __launch_bounds__(256, 1)
 k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *__restrict__ W,
           int M, int N, int K, int tiles_m, int total, int per_xcd, QkNorm qn) {
-    constexpr int TN = 256;
+    /* NA blocks of 16 output columns per wave: tiles of 256 rows x TN = 32 NA columns (256, 224 or 192), so that the
+     * launcher can pick the width whose grid fills the last round of the 256 CUs best. */
+    constexpr int TN = 32 * NA;
     constexpr int STAGE = (TN + DT) * TK;                      /* elements: W tile then x tile */
-    constexpr int NC = 8;                                      /* chunks of W (and of x) per thread and k tile: rows srow + 32 c */
+    constexpr int NCW = NA, NCX = 8, NCH = NCW + NCX;          /* 16 B chunks of W and of x per thread and k tile: rows srow + 32 c */
     extern __shared__ __align__(16) uint16_t dlds[];          /* two stages (and room for the epilogue) */
     const int work = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (work >= total) return;
@@ -524,13 +526,16 @@ k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *_
     const int band = work / (BAND * tiles_n), in_band = work - band * (BAND * tiles_n);
     const int band_rows = min(tiles_m - band * BAND, BAND);
     const int bm = band * BAND + in_band % band_rows, bn = in_band / band_rows;
-    const int m0 = bm * DT, n0 = bn * TN;
+    /* The last tile of a row or column of tiles is moved back so that it ends with the matrix: it overlaps its
+     * neighbour, and both write the same bits there (an output's products are summed in the same order whatever
+     * tile it is in). So no row is ever clamped and no store bounded. */
+    const int m0 = min(bm * DT, M - DT), n0 = min(bn * TN, N - TN);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
     const int wm = wave & 1, wn = wave >> 1;
 
-    /* staging: chunk tid % 8 of rows tid / 8 + 32 c; (row >> 1) & 7 is the same for all c. Whole tiles only
-     * (M and N multiples of 256), so no row is clamped and the 16 loads of a thread differ by uniform offsets. */
+    /* staging: chunk tid % 8 of rows tid / 8 + 32 c; (row >> 1) & 7 is the same for all c, and the loads of a
+     * thread differ by uniform offsets */
     const int srow = tid >> 3, schunk = tid & 7;
     const int st_off = srow * TK + 8 * (schunk ^ ((srow >> 1) & 7));
     const char *wt = reinterpret_cast<const char *>(W + (size_t)n0 * K), *xt = reinterpret_cast<const char *>(x + (size_t)m0 * K);   /* uniform tile bases */
@@ -538,24 +543,24 @@ k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *_
     uint32_t tile_b = 0;                                                        /* uniform: bytes of the k tile to fetch next */
     const uint32_t cstride = 64u * (uint32_t)K;                                 /* 32 rows, in bytes */
     const int nk = K / TK, nk_tiles = nk;
-    u32x4 wreg[2][NC], xreg[2][NC];                            /* two tiles on their way at any time */
+    u32x4 wreg[2][NCW], xreg[2][NCX];                          /* two tiles on their way at any time */
     int fetched = 0;                                           /* tiles requested so far; tile_b stays on the last tile at the end */
-    auto fetch_one = [&](int set, int c) {                     /* c < 8: chunk c of W, else chunk c - 8 of x */
-        if (c < NC) wreg[set][c] = *reinterpret_cast<const u32x4 *>(wt + (size_t)(tile_b + c * cstride) + lane_b);
-        else xreg[set][c - NC] = *reinterpret_cast<const u32x4 *>(xt + (size_t)(tile_b + (c - NC) * cstride) + lane_b);
+    auto fetch_one = [&](int set, int c) {                     /* c < NCW: chunk c of W, else chunk c - NCW of x */
+        if (c < NCW) wreg[set][c] = *reinterpret_cast<const u32x4 *>(wt + (size_t)(tile_b + c * cstride) + lane_b);
+        else xreg[set][c - NCW] = *reinterpret_cast<const u32x4 *>(xt + (size_t)(tile_b + (c - NCW) * cstride) + lane_b);
     };
     auto fetched_tile = [&]() { fetched++; tile_b += fetched < nk_tiles ? 2u * TK : 0u; };
     auto store_half = [&](int set, int stage, int c, int hi) {  /* 8 of the 16 bytes of chunk c */
         uint16_t *w_dst = dlds + stage * STAGE + st_off + 4 * hi;
-        const u32x4 v = c < NC ? wreg[set][c] : xreg[set][c - NC];
-        uint16_t *dst = c < NC ? w_dst + 32 * c * TK : w_dst + TN * TK + 32 * (c - NC) * TK;
+        const u32x4 v = c < NCW ? wreg[set][c] : xreg[set][c - NCW];
+        uint16_t *dst = c < NCW ? w_dst + 32 * c * TK : w_dst + TN * TK + 32 * (c - NCW) * TK;
         *reinterpret_cast<uint2 *>(dst) = hi ? make_uint2(v[2], v[3]) : make_uint2(v[0], v[1]);
     };
     auto store_one = [&](int set, int stage, int c) { store_half(set, stage, c, 0); store_half(set, stage, c, 1); };
 
-    f32x4 acc[8][8];                                           /* [a: 16 columns][b: 16 rows] */
+    f32x4 acc[NA][8];                                          /* [a: 16 columns][b: 16 rows] */
 #pragma unroll
-    for (int a = 0; a < 8; a++)
+    for (int a = 0; a < NA; a++)
 #pragma unroll
         for (int b = 0; b < 8; b++) acc[a][b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
@@ -563,18 +568,16 @@ k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *_
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
         const int slot = 8 * ((4 * ks + lg) ^ (li >> 1));
-        a_rd[ks] = (128 * wn + li) * TK + slot;
+        a_rd[ks] = (16 * NA * wn + li) * TK + slot;
         b_rd[ks] = TN * TK + (128 * wm + li) * TK + slot;
     }
 
-    /* Four steps of 32 MFMAs per k tile: k-step ks = step / 2, x blocks 4 (step % 2) .. + 3. The operands of a step
-     * are requested from the LDS before the products of the step before it are issued, across the tile boundary
-     * too. One barrier per tile, behind the products of step 2: by then every wave has written its share of tile
-     * kt + 1 (step 0) and has read the last operands of tile kt (step 2), so after it the stage of tile kt + 1 is
-     * complete and the stage of tile kt is free for tile kt + 2. The products are asm statements with the
-     * accumulators in AGPRs; the copies registers -> LDS of tile kt + 1 and the loads of tile kt + 2 stand between
-     * the products of step 0, one of each behind every second product. */
-    u32x4 av[2][8], bv[2][4];
+    /* Four steps of 4 NA MFMAs per k tile: k-step ks = step / 2, x blocks 4 (step % 2) .. + 3. The operands of a
+     * step are requested from the LDS during the step before it, across the tile boundary too. One barrier per
+     * tile, behind the products of step 2: by then every wave has written its share of tile kt + 1 and has read
+     * the last operands of tile kt, so after it the stage of tile kt + 1 is complete and the stage of tile kt is
+     * free for tile kt + 2. The products are asm statements with the accumulators in AGPRs. */
+    u32x4 av[2][NA], bv[2][4];
     auto read_a_one = [&](const uint16_t *stage, int ks, int a) {
         av[ks][a] = *reinterpret_cast<const u32x4 *>(&stage[a_rd[ks] + 16 * a * TK]);
     };
@@ -586,26 +589,26 @@ k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *_
 #pragma unroll
         for (int b = 0; b < 4; b++)
 #pragma unroll
-            for (int a = 0; a < 8; a++) {
+            for (int a = 0; a < NA; a++) {
                 asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[a][4 * half + b]) : "v"(av[ks][a]), "v"(bv[step & 1][b]));
-                between(8 * b + a);
+                between(NA * b + a);
             }
     };
 
 #pragma unroll
-    for (int c = 0; c < 2 * NC; c++) fetch_one(0, c);          /* tile 0 */
+    for (int c = 0; c < NCH; c++) fetch_one(0, c);             /* tile 0 */
     fetched_tile();
 #pragma unroll
-    for (int c = 0; c < 2 * NC; c++) store_one(0, 0, c);
+    for (int c = 0; c < NCH; c++) store_one(0, 0, c);
 #pragma unroll
-    for (int c = 0; c < 2 * NC; c++) fetch_one(1, c);          /* tiles 1 and 2 (or the last tile again) wait in the registers */
+    for (int c = 0; c < NCH; c++) fetch_one(1, c);             /* tiles 1 and 2 (or the last tile again) wait in the registers */
     fetched_tile();
 #pragma unroll
-    for (int c = 0; c < 2 * NC; c++) fetch_one(0, c);
+    for (int c = 0; c < NCH; c++) fetch_one(0, c);
     fetched_tile();
     lds_barrier();
 #pragma unroll
-    for (int a = 0; a < 8; a++) read_a_one(dlds, 0, a);
+    for (int a = 0; a < NA; a++) read_a_one(dlds, 0, a);
 #pragma unroll
     for (int b = 0; b < 4; b++) read_b_one(dlds, 0, b);
 
@@ -614,21 +617,28 @@ k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *_
         const uint16_t *cur = dlds + (kt & 1) * STAGE, *nxt = dlds + ((kt + 1) & 1) * STAGE;
         const int nstage = (kt + 1) & 1;
         /* At most one memory instruction behind a product: the wave issues in order, and what it issues between
-         * two products has to fit into the 12 cycles the matrix core still works on the first. Odd slots of steps 0
-         * and 1: tile kt + 1 registers -> LDS (chunk c behind product 4 c + 1) and tile kt + 3 -> registers (behind
-         * 4 c + 3); even slots: the operands of the next step, in the order its products use them. */
+         * two products has to fit into the 12 cycles the matrix core still works on the first. Even gaps: the
+         * operands of the next step in the order its products use them (4 x-blocks, and for an odd step the NA
+         * W-blocks of its k-step). Odd gaps of steps 0 - 2, 6 NA of them: the 3 NCH staging jobs in order, chunk by
+         * chunk two 8-byte copies registers -> LDS of tile kt + 1 and then the load of the same chunk of tile
+         * kt + 3 into the registers just freed; the few that do not fit (NA = 7: 45 jobs, 42 odd gaps) take the
+         * even gaps of step 2 behind its four reads. */
+        constexpr int ODD = 2 * NA;                             /* odd gaps per step */
+        auto staging_job = [&](int j) {
+            if (j >= 3 * NCH) return;
+            const int c = j / 3, part = j - 3 * c;
+            if (part < 2) store_half(set, nstage, c, part);
+            else fetch_one(set, c);
+        };
         auto slot = [&](int step, int i) {
-            if (step < 3 && (i & 1)) {                          /* odd slots of steps 0 - 2: 48 = 16 x (two halves, one load) */
-                const int j = 16 * step + (i >> 1), c = j / 3, part = j - 3 * c;
-                if (part < 2) store_half(set, nstage, c, part);
-                else fetch_one(set, c);
-            }
-            if ((i & 1) == 0) {
-                const int r = i >> 1;
+            const int r = i >> 1;
+            if (i & 1) {
+                if (step < 3) staging_job(ODD * step + r);
+            } else {
                 if (step == 0 && r < 4) read_b_one(cur, 1, r);
-                if (step == 1) { if (r < 4) read_b_one(cur, 2, r); else if (r < 12) read_a_one(cur, 1, r - 4); }
-                if (step == 2 && r < 4) read_b_one(cur, 3, r);
-                if (step == 3) { if (r < 4) read_b_one(nxt, 0, r); else if (r < 12) read_a_one(nxt, 0, r - 4); }
+                if (step == 1) { if (r < 4) read_b_one(cur, 2, r); else if (r < 4 + NA) read_a_one(cur, 1, r - 4); }
+                if (step == 2) { if (r < 4) read_b_one(cur, 3, r); else staging_job(3 * ODD + r - 4); }
+                if (step == 3) { if (r < 4) read_b_one(nxt, 0, r); else if (r < 4 + NA) read_a_one(nxt, 0, r - 4); }
             }
         };
         products(0, [&](int i) { slot(0, i); });
@@ -645,12 +655,12 @@ k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *_
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");                /* the last products have left the matrix core before the accumulators are read */
     lds_barrier();                                              /* the LDS is reused by the epilogue */
 
-    /* acc[a][b][r] = y[m0 + 128 wm + 16 b + li][n0 + 128 wn + 16 a + 4 lg + r] */
+    /* acc[a][b][r] = y[m0 + 128 wm + 16 b + li][n0 + 16 NA wn + 16 a + 4 lg + r] */
     constexpr int PER16 = 16 / (int)sizeof(OUT);
-    const int mw = m0 + 128 * wm, nw = n0 + 128 * wn;
+    const int mw = m0 + 128 * wm, nw = n0 + 16 * NA * wn;
     if constexpr (QKN) {
         /* the whole 256 x 256 bf16 tile in the LDS (128 KB), then a 16-lane row per (token, head) vector: see k_gemm_dma */
-        static_assert(sizeof(OUT) == 2, "bf16 projection only");
+        static_assert(sizeof(OUT) == 2 && NA == 8, "bf16 projection, tiles of two whole heads");
         if (n0 < qn.qk_cols) {
 #pragma unroll
             for (int b = 0; b < 8; b++)
@@ -712,7 +722,7 @@ k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *_
 #pragma unroll
                 for (int bb = 0; bb < 4; bb++)
 #pragma unroll
-                    for (int a = 0; a < 8; a++) {
+                    for (int a = 0; a < NA; a++) {
                         const int chunk = 4 * a + lg;
                         *reinterpret_cast<f32x4 *>(&buf[(16 * bb + li) * 128 + 4 * ((chunk & 16) | ((chunk ^ li) & 15))]) = acc[a][4 * half + bb];
                     }
@@ -721,7 +731,7 @@ k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *_
                     const int row = 2 * it + (lane >> 5), c = lane & 31;
                     f32x4 v = *reinterpret_cast<const f32x4 *>(&buf[row * 128 + 4 * ((c & 16) | ((c ^ row) & 15))]);
                     const int m = mw + 64 * half + row, n = nw + 4 * c;
-                    if (m < M && n < N) {
+                    if (c < 4 * NA) {
                         *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(y) + (size_t)m * N + n) = v;
                     }
                 }
@@ -731,7 +741,7 @@ k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *_
 #pragma unroll
             for (int b = 0; b < 8; b++)
 #pragma unroll
-                for (int a = 0; a < 8; a++) {
+                for (int a = 0; a < NA; a++) {
                     const int chunk = 2 * a + (lg >> 1);
                     *reinterpret_cast<uint2 *>(&buf[(16 * b + li) * 128 + 8 * (chunk ^ li) + 4 * (lg & 1)]) =
                         make_uint2(pack_bf16(acc[a][b][0], acc[a][b][1]), pack_bf16(acc[a][b][2], acc[a][b][3]));
@@ -741,7 +751,7 @@ k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *_
                 const int row = 4 * it + (lane >> 4), c = lane & 15;
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(&buf[row * 128 + 8 * (c ^ (row & 15))]);
                 const int m = mw + row, n = nw + 8 * c;
-                if (m < M && n < N) *reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(y) + (size_t)m * N + n) = v;
+                if (c < 2 * NA) *reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(y) + (size_t)m * N + n) = v;
             }
         }
         return;
@@ -751,7 +761,7 @@ k_gemm_w4(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *_
         const int m = mw + 16 * b + li;
         if (m >= M) continue;
 #pragma unroll
-        for (int a = 0; a < 8; a++) {
+        for (int a = 0; a < NA; a++) {
             const int n = nw + 16 * a + 4 * lg;
             if (n >= N) continue;
             f32x4 v = acc[a][b];
@@ -795,24 +805,41 @@ k_gemm_scalar(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_
     store4(y + i, v, 1);
 }
 
-template <typename OUT, bool QKN = false>
+template <typename OUT, int NA, bool QKN = false>
 int launch_gemm_w4(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, int N, int K, const QkNorm &qn = QkNorm{}) {
     static bool configured = false;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_w4<OUT, QKN>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_w4<OUT, NA, QKN>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, DMA_LDS_BYTES);
         if (e != hipSuccess) return (int)e;
         configured = true;
     }
-    const int tiles_m = M / DT, tiles_n = N / 256, total = tiles_m * tiles_n;
+    const int tiles_m = (M + DT - 1) / DT, tiles_n = (N + 32 * NA - 1) / (32 * NA), total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) / 8;
-    hipLaunchKernelGGL((k_gemm_w4<OUT, QKN>), dim3((unsigned)per_xcd * 8), dim3(256), DMA_LDS_BYTES, st, y, x, W, M, N, K,
+    hipLaunchKernelGGL((k_gemm_w4<OUT, NA, QKN>), dim3((unsigned)per_xcd * 8), dim3(256), DMA_LDS_BYTES, st, y, x, W, M, N, K,
                        tiles_m, total, per_xcd, qn);
     return (int)hipGetLastError();
 }
 
-/* Whole 256 x 256 tiles and an even number of k tiles: what the four-wave kernel takes. */
-static bool whole_tiles(int M, int N, int K) { return M % DT == 0 && N % 256 == 0 && K % (2 * TK) == 0; }
+/* What the four-wave kernel takes: at least one tile each way (its last tiles are moved back to end with the
+ * matrix, so the sizes need not be multiples of the tile) and an even number of k tiles. 16-byte stores. */
+static bool four_wave_shape(int M, int N, int K, size_t out_size) {
+    return M >= DT && N >= 256 && K % (2 * TK) == 0 && N % (16 / (int)out_size) == 0;
+}
+
+/* The tile width (32 NA columns) whose grid wastes least of its last round of 256 workgroups: time goes with
+ * rounds x width. 4608 x 9216 outputs: 648 tiles of 256 columns are 2.53 rounds, 756 of 224 are 2.95. */
+static int four_wave_width(int M, int N) {
+    const long tiles_m = (M + DT - 1) / DT;
+    int best = 8;
+    long best_cost = 0;
+    for (int na = 8; na >= 6; na--) {
+        const long tiles = tiles_m * ((N + 32 * na - 1) / (32 * na));
+        const long cost = ((tiles + 255) / 256) * na * (na == 8 ? 100 : 102);      /* the narrower tiles reuse operands a little less */
+        if (na == 8 || cost < best_cost) { best = na; best_cost = cost; }
+    }
+    return best;
+}
 
 template <typename OUT>
 int gemm(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, int N, int K) {
@@ -820,8 +847,14 @@ int gemm(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, in
     const bool aligned16 = ((uintptr_t)x & 15) == 0 && ((uintptr_t)W & 15) == 0;
     if (K > 0 && K % TK == 0 && aligned16 && M >= DT && N >= DT && (size_t)K * 2 * 8 < ((size_t)1 << 31)) {
         const ConvGeom none = {};
-        const int e = whole_tiles(M, N, K) ? launch_gemm_w4<OUT>(st, y, x, W, M, N, K)
-                                           : launch_gemm_dma<OUT, 256, false>(st, y, x, W, M, N, K, none);
+        int e;
+        if (four_wave_shape(M, N, K, sizeof(OUT)) && ((uintptr_t)y & 15) == 0) {
+            const int na = four_wave_width(M, N);
+            e = na == 8 ? launch_gemm_w4<OUT, 8>(st, y, x, W, M, N, K)
+              : na == 7 ? launch_gemm_w4<OUT, 7>(st, y, x, W, M, N, K) : launch_gemm_w4<OUT, 6>(st, y, x, W, M, N, K);
+        } else {
+            e = launch_gemm_dma<OUT, 256, false>(st, y, x, W, M, N, K, none);
+        }
         if (e) return e;
     } else if (K > 0 && K % 8 == 0 && aligned16) {
         /* 2 x 2 waves (128 x 128 tiles) measured best on the transformer shapes: 4 x 2 and 2 x 4 are
@@ -899,7 +932,8 @@ int iris_hip_linear_bf16_qknorm(void *stream, uint16_t *y, const uint16_t *x, co
         return -2;
     const ConvGeom none = {};
     const QkNorm qn = {wq, k_cols ? wk : wq, rope_cos, rope_sin, q_cols, q_cols + k_cols, eps, split_half};
-    if (whole_tiles(M, N, K)) return launch_gemm_w4<uint16_t, true>((hipStream_t)stream, y, x, W, M, N, K, qn);
+    if (M % DT == 0 && N % 256 == 0 && K % (2 * TK) == 0)          /* whole tiles: a tile holds two whole heads */
+        return launch_gemm_w4<uint16_t, 8, true>((hipStream_t)stream, y, x, W, M, N, K, qn);
     return launch_gemm_dma<uint16_t, 256, false, true>((hipStream_t)stream, y, x, W, M, N, K, none, qn);
 }
 
