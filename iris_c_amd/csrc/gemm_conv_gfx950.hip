@@ -841,22 +841,34 @@ static int four_wave_width(int M, int N) {
     return best;
 }
 
+/* Which kernel a linear layer takes, host arithmetic only: 3 = k_gemm_w4 with tiles of 32 na columns, 2 = k_gemm_dma,
+ * 1 = k_gemm_bf16, 0 = k_gemm_scalar. */
+struct GemmPlan { int kernel, na; };
+static GemmPlan plan_gemm(int M, int N, int K, int out_size, bool operands_aligned16, bool out_aligned16) {
+    if (K > 0 && K % TK == 0 && operands_aligned16 && M >= DT && N >= DT && (size_t)K * 2 * 8 < ((size_t)1 << 31)) {
+        if (four_wave_shape(M, N, K, (size_t)out_size) && out_aligned16) return {3, four_wave_width(M, N)};
+        return {2, 8};
+    }
+    if (K > 0 && K % 8 == 0 && operands_aligned16) return {1, 0};
+    return {0, 0};
+}
+
 template <typename OUT>
 int gemm(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W, int M, int N, int K) {
     if (M <= 0 || N <= 0) return 0;
     const bool aligned16 = ((uintptr_t)x & 15) == 0 && ((uintptr_t)W & 15) == 0;
-    if (K > 0 && K % TK == 0 && aligned16 && M >= DT && N >= DT && (size_t)K * 2 * 8 < ((size_t)1 << 31)) {
+    const GemmPlan plan = plan_gemm(M, N, K, (int)sizeof(OUT), aligned16, ((uintptr_t)y & 15) == 0);
+    if (plan.kernel == 3 || plan.kernel == 2) {
         const ConvGeom none = {};
         int e;
-        if (four_wave_shape(M, N, K, sizeof(OUT)) && ((uintptr_t)y & 15) == 0) {
-            const int na = four_wave_width(M, N);
-            e = na == 8 ? launch_gemm_w4<OUT, 8>(st, y, x, W, M, N, K)
-              : na == 7 ? launch_gemm_w4<OUT, 7>(st, y, x, W, M, N, K) : launch_gemm_w4<OUT, 6>(st, y, x, W, M, N, K);
+        if (plan.kernel == 3) {
+            e = plan.na == 8 ? launch_gemm_w4<OUT, 8>(st, y, x, W, M, N, K)
+              : plan.na == 7 ? launch_gemm_w4<OUT, 7>(st, y, x, W, M, N, K) : launch_gemm_w4<OUT, 6>(st, y, x, W, M, N, K);
         } else {
             e = launch_gemm_dma<OUT, 256, false>(st, y, x, W, M, N, K, none);
         }
         if (e) return e;
-    } else if (K > 0 && K % 8 == 0 && aligned16) {
+    } else if (plan.kernel == 1) {
         /* 2 x 2 waves (128 x 128 tiles) measured best on the transformer shapes: 4 x 2 and 2 x 4 are
          * 5-8 % slower on the wide projections, 4 x 1 and 2 x 1 15-30 % slower. */
         constexpr int WM = 2, WN = 2, TM = 64 * WM, TN = 64 * WN;
@@ -907,6 +919,13 @@ k_add_bias_rows(float *__restrict__ y, const float *__restrict__ bias, int cols,
 }  // namespace
 
 extern "C" {
+
+/* The kernel a linear layer of these sizes takes (aligned operands): plan[0] = 3 four waves, 2 eight waves with
+ * direct loads, 1 the 128 x 128 kernel, 0 scalar; plan[1] = columns of a tile of the four-wave kernel. No GPU needed. */
+void iris_hip_linear_plan(int rows, int in, int out, int out_bytes, int *plan) {
+    const GemmPlan p = plan_gemm(rows, out, in, out_bytes, true, true);
+    plan[0] = p.kernel; plan[1] = p.kernel == 3 ? 32 * p.na : 0;
+}
 
 int iris_hip_linear_f32(void *stream, float *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out) {
     return gemm<float>((hipStream_t)stream, y, x, W, rows, out, in);

@@ -118,6 +118,11 @@ int iris_hip_group_norm_static(void *stream, float *out, const float *in, const 
 int iris_hip_linear_f32(void *stream, float *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out);
 int iris_hip_linear_bf16(void *stream, uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out);
 /* -2 = shape not taken, nothing enqueued */
+/* Which kernel a linear layer of these sizes takes with aligned operands, host arithmetic only: plan[0] = 3 the
+ * four-wave 256-row tiles, 2 the eight-wave ones, 1 the 128 x 128 kernel, 0 the scalar kernel; plan[1] = the tile width
+ * of the four-wave kernel (256, 224 or 192 columns). */
+void iris_hip_linear_plan(int rows, int in, int out, int out_bytes, int *plan);
+
 int iris_hip_linear_bf16_qknorm(void *stream, uint16_t *y, const uint16_t *x, const uint16_t *W, int rows, int in, int out,
                                 int q_cols, int k_cols, const float *wq, const float *wk, const float *rope_cos,
                                 const float *rope_sin, float eps, int split_half);

@@ -1,6 +1,6 @@
-"""The attention launcher's choice of kernel and grid is host arithmetic (iris_hip_fa_hd128_plan): which workgroup
-shape a problem gets, and for the two-size grid how many workgroups of 256 and of 192 queries per head. Runs without a
-GPU: the library loads, nothing is launched."""
+"""The launchers' choices are host arithmetic: which workgroup shape an attention problem gets, and for the two-size
+grid how many workgroups of 256 and of 192 queries per head (iris_hip_fa_hd128_plan); which GEMM kernel and tile width
+a linear layer gets (iris_hip_linear_plan). Runs without a GPU: the library loads, nothing is launched."""
 import ctypes as C
 
 import pytest
@@ -57,3 +57,29 @@ def test_two_size_grids_cover_every_query_and_never_lose_to_one_size(plan, heads
 def test_exact_rounds_keep_one_size(plan):
     for heads, seq in ((16, 4096), (32, 2048), (8, 8192), (32, 4096), (30, 4352)):
         assert plan(seq, seq, heads)["kind"] == 0, (heads, seq)
+
+
+# ------------------------------------------------------------------ the linear layers' kernel choice
+@pytest.fixture(scope="module")
+def linear_plan():
+    lib = C.CDLL(iris_c_amd.LIB_PATH)
+    lib.iris_hip_linear_plan.argtypes = [C.c_int] * 4 + [C.POINTER(C.c_int)]
+    lib.iris_hip_linear_plan.restype = None
+
+    def call(rows, k, out, out_bytes=2):
+        p = (C.c_int * 2)()
+        lib.iris_hip_linear_plan(rows, k, out, out_bytes, p)
+        return p[0], p[1]
+    return call
+
+
+def test_linear_layers_of_the_models_take_the_four_wave_kernel_in_the_width_that_fills_the_rounds(linear_plan):
+    assert linear_plan(4608, 3072, 9216) == (3, 224)        # 756 tiles = 2.95 rounds of 256 CUs (648 of 256 columns: 2.53)
+    assert linear_plan(4608, 3072, 3072) == (3, 224)        # 252 tiles: one round (216 of 256 columns: also one, but wider)
+    assert linear_plan(4608, 3072, 27648) == (3, 256)       # 1944 tiles = 7.6 rounds; narrower tiles need 9 or 11
+    assert linear_plan(4608, 3072, 18432)[1] in (224, 192)  # 1296 tiles of 256 columns are 5.06 rounds
+    for rows, k, out in ((300, 128, 258), (257, 64, 257), (512, 192, 256)):
+        assert linear_plan(rows, k, out)[0] == 2             # k not a multiple of 128, or rows of 2 bytes not 16-byte aligned
+    assert linear_plan(700, 256, 1000) == (3, 256) or linear_plan(700, 256, 1000)[0] == 3
+    assert linear_plan(64, 128, 64)[0] == 1 and linear_plan(37, 27, 19)[0] == 0
+    assert linear_plan(512, 256, 258, 4)[0] == 2             # f32 rows of 258 columns cannot take 16-byte stores
