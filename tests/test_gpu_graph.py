@@ -36,7 +36,7 @@ class Graphs:
         return run
 
 
-@pytest.mark.parametrize("maker", [W.c1, W.c4, lambda: W.c2(shrink=4)], ids=["c1", "c4", "c2-shrunk"])
+@pytest.mark.parametrize("maker", [W.c1, W.c4, lambda: W.c2(shrink=4), W.c2], ids=["c1", "c4", "c2-shrunk", "c2-two-size-grid"])
 def test_step_replayed_from_a_graph_equals_the_eager_step(maker):
     case = maker()
     dev, g = Dev(), Graphs()
