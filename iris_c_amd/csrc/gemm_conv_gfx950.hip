@@ -822,9 +822,11 @@ int launch_gemm_w4(hipStream_t st, OUT *y, const uint16_t *x, const uint16_t *W,
 }
 
 /* What the four-wave kernel takes: at least one tile each way (its last tiles are moved back to end with the
- * matrix, so the sizes need not be multiples of the tile) and an even number of k tiles. 16-byte stores. */
+ * matrix, so the sizes need not be multiples of the tile), an even number of k tiles, 16-byte stores, and tiles
+ * of less than 4 GB. */
 static bool four_wave_shape(int M, int N, int K, size_t out_size) {
-    return M >= DT && N >= 256 && K % (2 * TK) == 0 && N % (16 / (int)out_size) == 0;
+    return M >= DT && N >= 256 && K % (2 * TK) == 0 && N % (16 / (int)out_size) == 0 &&
+           (size_t)K * 2 * (DT + 32) < ((size_t)1 << 32);             /* a thread's byte offsets into a tile are 32-bit */
 }
 
 /* The tile width (32 NA columns) whose grid wastes least of its last round of 256 workgroups: time goes with
