@@ -488,17 +488,17 @@ k_gemm_dma(OUT *__restrict__ y, const uint16_t *__restrict__ x, const uint16_t *
         }
     }
 }
-/* ---- the same 256 x 256 x 64 tiles on FOUR waves, one per SIMD with the whole register file ----
+/* ---- tiles of 256 rows x 256, 224 or 192 columns x 64 on FOUR waves, one per SIMD with the whole register file ----
  *
  * For M, N >= 256 and K a multiple of 128. Each wave owns 128 rows x 16 NA columns = NA x 8 accumulator
  * blocks, up to 256 registers that live in AGPRs (the products are asm statements, so that they stay there),
- * so an operand read from the LDS feeds eight products: 32 reads per 128 MFMAs and k tile, two thirds of the LDS
- * traffic of the 8-wave kernel. A wave that is alone on its SIMD has nobody to hide its other instructions behind:
+ * so an operand read from the LDS feeds NA or eight products: with NA = 8, 32 reads per 128 MFMAs and k tile, two
+ * thirds of the LDS traffic of the 8-wave kernel. A wave that is alone on its SIMD has nobody to hide its other instructions behind:
  * it issues in order, and what stands between two products must fit into the 12 cycles the matrix core still
  * works on the first. Hence
  *  - the tiles are staged through registers (a direct HBM -> LDS load blocks the issuing wave for about 100
- *    cycles): 16 loads of 16 B per thread and k tile, two tiles ahead (two register sets), each written to the
- *    LDS as two 8-byte halves (a 16-byte LDS write takes longer to issue than the gap: 1265 -> 1302 TFLOP/s);
+ *    cycles): NA + 8 loads of 16 B per thread and k tile, two tiles ahead (two register sets), each written to
+ *    the LDS as two 8-byte halves (a 16-byte LDS write takes longer to issue than the gap: 1265 -> 1302 TFLOP/s);
  *  - every gap between two products holds at most one memory instruction: odd gaps of steps 0 - 2 the copies
  *    registers -> LDS of tile kt + 1 and the loads of tile kt + 3, even gaps the operand reads of the next step
  *    (all of them bunched at the step boundaries: 1160 TFLOP/s; two and a load per fourth gap: 1230; one per gap:
