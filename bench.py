@@ -64,15 +64,47 @@ PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E peak
 TRAFFIC_PROFILE = os.path.join("profiles", "k_fa_fwd_hd128__c2__hbm_traffic.txt")
 
 
+ATTENTION_SOURCE = os.path.join("iris_c_amd", "csrc", "fa_fwd_gfx950.hip")
+
+
+def source_sha256(rel=ATTENTION_SOURCE):
+    import hashlib
+    try:
+        return hashlib.sha256(open(os.path.join(ROOT, rel), "rb").read()).hexdigest()[:16]
+    except OSError:
+        return None
+
+
 def traffic_on_file():
-    """(bytes per launch, source) from the line 'total_bytes_per_launch: N' of the committed counter summary."""
+    """(bytes per launch, source file, stale) from the committed counter summary: the line
+    'total_bytes_per_launch: N', and 'kernel_source_sha256: H', the hash of the kernel source the counters were taken
+    on; stale = that hash is not the hash of the kernel source in this tree."""
+    nbytes, sha = None, None
     try:
         for line in open(os.path.join(ROOT, TRAFFIC_PROFILE)):
             if line.startswith("total_bytes_per_launch:"):
-                return int(line.split(":")[1].strip().replace(",", "")), TRAFFIC_PROFILE
+                nbytes = int(line.split(":")[1].strip().replace(",", ""))
+            if line.startswith("kernel_source_sha256:"):
+                sha = line.split(":")[1].strip()
     except OSError:
-        pass
-    return None, None
+        return None, None, None
+    return nbytes, TRAFFIC_PROFILE, sha != source_sha256()
+
+
+def attention_kernel_name(lib, c):
+    """The __global__ function an iris_dev_attention call of configuration c launches, from the launcher's own
+    planner (host arithmetic, nothing launched)."""
+    plan = (C.c_int * 5)()
+    lib.iris_hip_fa_hd128_plan.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int)]
+    lib.iris_hip_fa_hd128_plan.restype = None
+    lib.iris_hip_fa_hd128_plan(c["seq"], c["seq"], c["heads"], int(c["causal"]), plan)
+    flags = f"{'true' if c['causal'] else 'false'}, {'true' if c['key_mask'] is not None else 'false'}"
+    kind, waves, nb = plan[0], plan[1], plan[2]
+    if kind == 1:
+        return f"k_fa_fwd_hd128_two_sizes<{flags}>", {"workgroups_of_256_queries_per_head": plan[3], "workgroups_of_192_queries_per_head": plan[4]}
+    if kind == 2:
+        return f"k_fa_short_hd128<4, {flags}>", {}
+    return f"k_fa_fwd_hd128<{waves}, {nb}, {flags}>", {"queries_per_workgroup": 16 * nb * waves}
 
 NORM_ROPE_PROFILE = os.path.join("profiles", "k_norm_rope_hd128__c2__kernel_trace.txt")
 
@@ -198,6 +230,7 @@ class Resident:
         self.bufs = [dev.to_device(c["buf"]) for _ in range(copies)]
         self.out = self.lib.iris_dev_alloc(c["seq"] * c["ldo"] * 2)
         self.wq, self.wk = dev.to_device(c["wq"]), dev.to_device(c["wk"])
+        self.wq2, self.wk2 = dev.to_device(c["wq"][::-1].copy()), dev.to_device(c["wk"][::-1].copy())   # the image stream's pair
         self.cos, self.sin = dev.to_device(c["cos"]), dev.to_device(c["sin"])
         self.mask = dev.to_device(c["key_mask"]) if c["key_mask"] is not None else None
         assert self.out and all(self.bufs)
@@ -234,6 +267,37 @@ class Resident:
         """The same work with the library's one-launch Q+K normalisation (an addition to the reference API)."""
         self.norm_qk(i); self.attention(i)
 
+    # The double-stream block (reference iris_transformer_flux.c:3786-3804): text rows [0, txt) and image rows
+    # [txt, seq) of the joint q | k | v rows are normalised separately, each stream with its own weight pair and the
+    # tables offset to its first row; then one attention over all rows.
+    def _streams(self, txt):
+        return ((0, txt, self.wq, self.wk), (txt, self.c["seq"] - txt, self.wq2, self.wk2))
+
+    def norm_double_stream(self, i, txt):
+        """four launches, as the reference issues them"""
+        c = self.c
+        for first, n, wq, wk in self._streams(txt):
+            qkv = self.bufs[i % len(self.bufs)] + 2 * first * c["ldi"]
+            rc, rs = _vp(self.cos + 4 * first * 64), _vp(self.sin + 4 * first * 64)
+            self.lib.iris_dev_head_norm_rope(_vp(qkv), c["ldi"], wq, rc, rs, n, c["heads"], c["hd"], c["eps"], 0)
+            self.lib.iris_dev_head_norm_rope(_vp(qkv + 2 * c["q_dim"]), c["ldi"], wk, rc, rs, n, c["kv_heads"], c["hd"], c["eps"], 0)
+
+    def norm_double_stream_qk(self, i, txt):
+        """one Q+K launch per stream"""
+        c = self.c
+        for first, n, wq, wk in self._streams(txt):
+            qkv = self.bufs[i % len(self.bufs)] + 2 * first * c["ldi"]
+            rc, rs = _vp(self.cos + 4 * first * 64), _vp(self.sin + 4 * first * 64)
+            self.lib.iris_dev_head_norm_rope_qk(_vp(qkv), _vp(qkv + 2 * c["q_dim"]), c["ldi"], wq, wk, rc, rs, n, c["heads"],
+                                                c["kv_heads"], c["hd"], c["eps"], 0)
+
+    def norm_double_stream_one(self, i, txt):
+        """one launch for both streams and both tensors"""
+        c = self.c
+        self.lib.iris_dev_head_norm_rope_qk_streams(self.col(i, 0), self.col(i, c["q_dim"]), c["ldi"], self.wq, self.wk, self.wq2,
+                                                    self.wk2, txt, self.cos, self.sin, c["seq"], c["heads"], c["kv_heads"],
+                                                    c["hd"], c["eps"], 0)
+
     def attention_qnorm(self, i):
         c = self.c
         self.lib.iris_dev_attention_qnorm(self.out, c["ldo"], self.col(i, 0), self.col(i, c["q_dim"]),
@@ -247,7 +311,7 @@ class Resident:
         self.norm_k(i); self.attention_qnorm(i)
 
     def free(self):
-        for p in self.bufs + [self.out, self.wq, self.wk, self.cos, self.sin] + ([self.mask] if self.mask else []):
+        for p in self.bufs + [self.out, self.wq, self.wk, self.wq2, self.wk2, self.cos, self.sin] + ([self.mask] if self.mask else []):
             self.lib.iris_dev_free(p)
 
 
@@ -435,6 +499,8 @@ def microbench_lib():
     mb.iris_mb_mfma_data16.argtypes = [_vp, _vp, _vp, C.c_int, C.c_int]
     mb.iris_mb_copy.argtypes = [_vp, _vp, _vp, C.c_size_t]
     mb.iris_mb_rmw.argtypes = [_vp, _vp, C.c_size_t]
+    mb.iris_mb_read.argtypes = [_vp, _vp, C.c_size_t, _vp]
+    mb.iris_mb_write.argtypes = [_vp, _vp, C.c_size_t]
     return mb
 
 
@@ -541,10 +607,35 @@ def machine_ceilings(dev, hip, stream):
     assert all(ring)
     settle(lib, lambda i: mb.iris_mb_rmw(stream, _vp(ring[i % 24]), small), 20)
     rw_small = min(event_time(hip, stream, lambda i: mb.iris_mb_rmw(stream, _vp(ring[i % 24]), small), 48) for _ in range(3))
+    # Yardsticks that are not this library's kernels or shapes: the runtime's own device-to-device copy
+    # (hipMemcpyDtoDAsync on the library's stream), a read-only and a write-only stream; at 1 GiB and at the volume of
+    # one fused Q+K norm+rope call of the bench workload (54 MiB of rows) on the rotating buffers.
+    hip.rt.hipMemcpyDtoDAsync.argtypes = [_vp, _vp, C.c_size_t, _vp]
+    dtod = lambda dst, src, nbytes: hip.rt.hipMemcpyDtoDAsync(dst, src, nbytes, stream)
+    assert dtod(b, a, n) == 0
+    lib.iris_dev_sync()
+    dd = min(event_time(hip, stream, lambda i: dtod(b, a, n), 2) for _ in range(3))
+    rd = min(event_time(hip, stream, lambda i: mb.iris_mb_read(stream, a, n, sink), 2) for _ in range(3))
+    wr = min(event_time(hip, stream, lambda i: mb.iris_mb_write(stream, b, n), 2) for _ in range(3))
+    pair = lambda i: (_vp(ring[(2 * i) % 24]), _vp(ring[(2 * i + 1) % 24]))
+    dd_small = min(event_time(hip, stream, lambda i: dtod(*pair(i), small), 48) for _ in range(3))
+    cp_small = min(event_time(hip, stream, lambda i: mb.iris_mb_copy(stream, *pair(i), small), 48) for _ in range(3))
+    rd_small = min(event_time(hip, stream, lambda i: mb.iris_mb_read(stream, _vp(ring[i % 24]), small, sink), 48) for _ in range(3))
+    wr_small = min(event_time(hip, stream, lambda i: mb.iris_mb_write(stream, _vp(ring[i % 24]), small), 48) for _ in range(3))
     dev.check()
     for p in [sink, a, b, ops] + ring:
         lib.iris_dev_free(p)
-    return {"inplace_update_27mib_cold_us": round(rw_small * 1e3, 2),
+    yard = {"hip_memcpy_dtod_1gib_gbps": round(2 * n / dd / 1e6, 1), "read_only_1gib_gbps": round(n / rd / 1e6, 1),
+            "write_only_1gib_gbps": round(n / wr / 1e6, 1),
+            "hip_memcpy_dtod_27mib_cold_gbps": round(2 * small / dd_small / 1e6, 1),
+            "hip_memcpy_dtod_27mib_cold_us": round(dd_small * 1e3, 2),
+            "copy_27mib_cold_gbps": round(2 * small / cp_small / 1e6, 1), "copy_27mib_cold_us": round(cp_small * 1e3, 2),
+            "read_only_27mib_cold_gbps": round(small / rd_small / 1e6, 1), "read_only_27mib_cold_us": round(rd_small * 1e3, 2),
+            "write_only_27mib_cold_gbps": round(small / wr_small / 1e6, 1), "write_only_27mib_cold_us": round(wr_small * 1e3, 2),
+            "note": "bytes counted read + written for the copies, one direction for the one-way streams; 27 MiB series "
+                    "over 24 rotating buffers (648 MiB > the Infinity Cache), back-to-back launches between two events"}
+    return {"streaming_yardsticks": yard,
+            "inplace_update_27mib_cold_us": round(rw_small * 1e3, 2),
             "inplace_update_27mib_cold_gbps": round(2 * small / rw_small / 1e6, 1),
             "mfma_only_tflops": round(mfma, 1), "mfma_only_frac_of_peak": round(mfma / PEAK_BF16_TFLOPS, 4),
             "mfma_only_normal_data_tflops": round(mfma_data, 1),
@@ -714,13 +805,40 @@ def main():
         lib.iris_dev_sync()
         qnorm_ms = (time.perf_counter() - t0) / args.steps * 1e3
 
+    # the double-stream block's call pattern: four norm launches on row sub-ranges (512 text rows, 4096 image rows; Q
+    # and K each; two weight pairs) + attention; the same with one Q+K launch per stream, and with one launch in all
+    double = None
+    if not args.no_variants:
+        txt = c2["layout"][0]
+        double = {}
+        for key, norm in (("four_norm_launches", res.norm_double_stream), ("one_qk_launch_per_stream", res.norm_double_stream_qk),
+                          ("one_norm_launch", res.norm_double_stream_one)):
+            def step(i, norm=norm):
+                norm(i, txt); res.attention(i)
+            for i in range(args.warmup):
+                step(i)
+            lib.iris_dev_sync()
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                step(i)
+            lib.iris_dev_sync()
+            ms = (time.perf_counter() - t0) / args.steps * 1e3
+            n_ms = event_time(hip, stream, lambda i, norm=norm: norm(i, txt), max(args.steps, 2 * copies))
+            double[key] = {"ms_per_step": round(ms, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 2),
+                           "norm_launches_us": round(n_ms * 1e3, 2)}
+        dev.check()
+        double["note"] = ("reference iris_transformer_flux.c:3786-3804: per stream (512 text rows, 4096 image rows) norm+rope on Q "
+                          "and on K of the joint rows with the stream's own weights, then one attention over all 4608 rows; "
+                          "norm_launches_us = the norm launches alone, back to back over rotating (cold) rows")
+
     # dominant kernel in its place in the step: events around the attention launch of every step (Q and K rows
     # just rewritten by the two norm calls, V rows not touched since the buffer's last turn)
     att = per_launch_times(hip, stream, res.attention, max(args.steps, 10),
                            before=lambda i: (res.norm_q(i), res.norm_k(i)))
     att_ms = float(np.mean(att))
     att_single = single_launch_ms(hip, stream, lib, res.attention)
-    traffic, traffic_source = traffic_on_file()
+    traffic, traffic_source, traffic_stale = traffic_on_file()
+    kernel_name, kernel_grid = attention_kernel_name(lib, c2)
     # bandwidth-bound kernel: back-to-back launches over rotating buffers (cold) and one buffer (warm)
     reps = max(args.steps, 2 * copies)
     nr_q_ms = event_time(hip, stream, res.norm_q, reps)
@@ -748,10 +866,12 @@ def main():
         "step_with_q_norm_in_attention": None if qnorm_ms is None else {
             "ms_per_step": round(qnorm_ms, 4), "tflops": round(flops / (qnorm_ms * 1e-3) / 1e12, 2),
             "note": "two launches: iris_dev_head_norm_rope on K + iris_dev_attention_qnorm"},
-        "roofline": {"kernel": "k_fa_fwd_hd128", "bound": "mfma", "achieved": round(flops / (att_ms * 1e-3) / 1e12, 2),
+        "step_double_stream": double,
+        "roofline": {"kernel": kernel_name, "kernel_grid": kernel_grid, "kernel_source_sha256": source_sha256(),
+                     "bound": "mfma", "achieved": round(flops / (att_ms * 1e-3) / 1e12, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / (att_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
                      "traffic": traffic, "traffic_unit": "bytes per launch, hardware counters of a separate profiler run",
-                     "traffic_source": traffic_source,
+                     "traffic_source": traffic_source, "traffic_source_stale": traffic_stale,
                      "algorithmic_bytes": 4 * c2["seq"] * c2["q_dim"] * 2, "launch_ms": round(att_ms, 4),
                      "launch_ms_median": round(float(np.median(att)), 4), "launch_ms_min": round(float(np.min(att)), 4),
                      "single_launch_ms": round(att_single, 4),

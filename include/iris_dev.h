@@ -154,6 +154,19 @@ void iris_dev_head_norm_rope_qk(uint16_t *xq, uint16_t *xk, int ld,
                                 int seq, int q_heads, int k_heads, int head_dim,
                                 float eps, int split_half);
 
+/* The FOUR calls of a double-stream block (iris_transformer_flux.c:3796-3803: text rows and image rows of the joint
+ * q | k | v buffer, Q and K each, every stream with its own weight pair, tables offset to the stream's first row)
+ * as ONE launch over the joint rows: rows [0, rows_a) of xq / xk take (wq_a, wk_a), rows [rows_a, seq) take
+ * (wq_b, wk_b); row s of the tables belongs to row s of the joint sequence. Same result as
+ *     iris_dev_head_norm_rope(xq, ld, wq_a, cos, sin, rows_a, q_heads, ...);   ..(xk, ld, wk_a, ...)
+ *     iris_dev_head_norm_rope(xq + rows_a * ld, ld, wq_b, cos + rows_a * head_dim / 2, sin + ..., seq - rows_a, ...);
+ *     ..(xk + rows_a * ld, ld, wk_b, ...)
+ * bit for bit. The 512-row text calls alone are launch-bound (6.5 MB each). */
+void iris_dev_head_norm_rope_qk_streams(uint16_t *xq, uint16_t *xk, int ld,
+                                        const float *wq_a, const float *wk_a, const float *wq_b, const float *wk_b,
+                                        int rows_a, const float *rope_cos, const float *rope_sin,
+                                        int seq, int q_heads, int k_heads, int head_dim, float eps, int split_half);
+
 /* iris_dev_attention with the Q half of the normalisation folded in: the result is what
  *     iris_dev_head_norm_rope(q, ldi, wq, rope_cos, rope_sin, seq_q, heads, head_dim, eps, split_half);
  *     iris_dev_attention(out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, head_dim, scale, causal, key_mask);

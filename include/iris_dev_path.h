@@ -5,7 +5,7 @@
  * backend object (iris_cuda.cu:117-230 for setup and memory, :456-1200 for the other operators) -- and takes
  * only the two hot-path operators from here. The archive defines
  *     iris_dev_head_norm_rope, iris_dev_attention                     (reference iris_dev.h:74-92)
- *     iris_dev_head_norm_rope_qk, iris_dev_attention_qnorm,
+ *     iris_dev_head_norm_rope_qk, iris_dev_head_norm_rope_qk_streams, iris_dev_attention_qnorm,
  *     iris_dev_last_error, iris_dev_last_kernel                       (additions, see iris_dev.h)
  * and the two entries below, and none of the other symbols of iris_dev.h, so it links next to a backend that
  * defines those itself.

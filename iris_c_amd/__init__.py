@@ -50,6 +50,7 @@ ABI = {
     "iris_dev_group_norm_noalloc": (None, [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _i]),
     "iris_dev_upsample2x": (None, [_vp, _vp, _i, _i, _i]),
     "iris_dev_head_norm_rope_qk": (None, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i]),
+    "iris_dev_head_norm_rope_qk_streams": (None, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _i]),
     "iris_dev_stream": (_vp, []),
     "iris_dev_last_error": (_i, []),
     "iris_dev_last_kernel": (C.c_char_p, []),

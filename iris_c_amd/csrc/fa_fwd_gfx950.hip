@@ -463,6 +463,19 @@ fa_walk_hd128(uint16_t *__restrict__ lds, uint16_t *__restrict__ out, int ldo, c
         }
     }
 
+    /* A wave whose queries all lie behind the end of the sequence (the last workgroup of a head when seq_q is not a
+     * multiple of the workgroup's queries: 4608 = 10 x 256 + 11 x 192 - 64) multiplies nothing. It still fetches its
+     * share of every tile and passes the same barriers as the others: one per group of tiles, as the loop below. */
+    if (wq0 >= seq_q) {                                  /* wave-uniform */
+        for (int g0 = 0, half = 0; g0 < ntiles_run; g0 += GROUP, half ^= 1) {
+#pragma unroll
+            for (int t = 0; t < GROUP; t++) request(g0 + GROUP + t, (half ^ 1) * GROUP + t);
+            wait_vmcnt<0>();
+            lds_barrier();
+        }
+        return;
+    }
+
     for (int g0 = 0, half = 0; g0 < ntiles_run; g0 += GROUP, half ^= 1) {
 #pragma unroll
       for (int h = 0; h < GROUP; h++) {
@@ -735,6 +748,11 @@ k_fa_fwd_hd128_two_sizes(uint16_t *__restrict__ out, int ldo, const uint16_t *__
         two_blocks = wave < 4;
         wq0 = two_blocks ? q0 + 32 * wave : q0 + 128 + 16 * (wave - 4);
     }
+    /* Waves 0-3 and 4-7 of a 192-query workgroup run two instantiations of the walk and meet at its barriers.
+     * INVARIANT: every barrier of fa_walk_hd128 is passed the same number of times by both, i.e. no barrier may sit
+     * under a condition that depends on NB or on the wave's own queries (wq0) -- the tile counts ntiles / ntiles_run
+     * depend on the workgroup's q0, bm and the key mask only, and the path of a wave without queries in the sequence
+     * passes one barrier per group like the main loop. A violation would hang the GPU, not fail a test. */
     if (two_blocks)
         fa_walk_hd128<8, 2, 2, CAUSAL, MASK>(lds, out, ldo, q, k, v, ldi, seq_q, seq_k, head, head / kv_group, q0, bm, wq0,
                                              scale_log2, key_mask, qnorm);
@@ -814,7 +832,12 @@ k_fa_short_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict
             }
         }
     };
-    /* K tile `it` as A operands: key block mb, k-step ks -> key 16 mb + li, dims 32 ks + 8 lg .. + 7 */
+    /* K tile `it` as A operands: key block mb, k-step ks -> key 16 mb + li, dims 32 ks + 8 lg .. + 7.
+     * The waits further down count on EXACTLY 16 loads per request_k and 16 per request_v, completing in order, and
+     * on no other vector-memory load between a request and its wait (wait_vmcnt<16> = "everything but the newest 16").
+     * The compiler does not know that ka is pending between request and wait: nothing may read, copy or spill ka
+     * there. tests/test_gpu_attention.py::test_keys_split_over_the_waves_of_a_workgroup holds this kernel against
+     * the oracle on causal, masked and ragged calls and would catch a toolchain that breaks either assumption. */
     u32x4 ka[4][4];
     auto request_k = [&](int it) {
 #pragma unroll
@@ -1053,7 +1076,24 @@ k_fa_short_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict
 
 template <int W, int NB> constexpr size_t stage_bytes() { return (W * NB >= 12 ? 4 : 2) * STAGE * sizeof(uint16_t); }
 constexpr size_t LDS_MAX = 160 * 1024;
-constexpr int CUS = 256;
+
+/* Compute units of the current device (256 on an MI355X in its single-partition mode); 256 where no device answers,
+ * so that the planner can be exercised on a machine without a GPU. The costs further down were fitted on 256 CUs in
+ * 8 XCDs: another SKU or partition mode changes the rounds through this count, the cost constants want a re-fit. */
+int cu_count() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount >= 8)
+            n = prop.multiProcessorCount;
+        else {
+            (void)hipGetLastError();
+            n = 256;
+        }
+    }
+    return n;
+}
 
 template <int W, int NB, bool C, bool M>
 int launch(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
@@ -1181,7 +1221,7 @@ static long two_sizes_cost(long n_full, long n_tail) {
     long worst = 0;
     for (long s = 0; s < 4; s++) {
         const long full = fx > s ? (fx - s + 3) / 4 : 0, both = fx + tx > s ? (fx + tx - s + 3) / 4 : 0;
-        const long c = makespan(full, both - full, 78, CUS / XCDS / 4);
+        const long c = makespan(full, both - full, 78, cu_count() / XCDS / 4);
         if (c > worst) worst = c;
     }
     return worst;
@@ -1214,6 +1254,7 @@ static FaPlan plan_hd128(int seq_q, int seq_k, int heads, int causal) {
      * however few CUs it uses; a round of 128-query workgroups costs 1.1 when some CU gets two of them and 0.6
      * when none does (one wave per SIMD runs faster than two, not twice as fast). Constants measured on 16 to 48
      * heads, 256 .. 12800 tokens, clocks settled. */
+    const long CUS = cu_count();
     const long waves16 = (long)((seq_q + 15) / 16) * heads;
     if (waves16 <= 8 * CUS) {
         const int w = waves16 <= CUS ? 1 : waves16 <= 640 ? 2 : waves16 <= 4 * CUS ? 4 : 8;

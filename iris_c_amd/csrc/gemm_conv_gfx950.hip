@@ -953,7 +953,7 @@ int iris_hip_linear_bf16_qknorm(void *stream, uint16_t *y, const uint16_t *x, co
         return -2;
     const ConvGeom none = {};
     const QkNorm qn = {wq, k_cols ? wk : wq, rope_cos, rope_sin, q_cols, q_cols + k_cols, eps, split_half};
-    if (M % DT == 0 && N % 256 == 0 && K % (2 * TK) == 0)          /* whole tiles: a tile holds two whole heads */
+    if (M % DT == 0 && N % 256 == 0 && four_wave_shape(M, N, K, 2))   /* whole tiles: a tile holds two whole heads */
         return launch_gemm_w4<uint16_t, 8, true>((hipStream_t)stream, y, x, W, M, N, K, qn);
     return launch_gemm_dma<uint16_t, 256, false, true>((hipStream_t)stream, y, x, W, M, N, K, none, qn);
 }

@@ -22,6 +22,14 @@ int iris_hip_norm_rope_hd128(void *stream, uint16_t *xq, uint16_t *xk, int ld,
                              const float *rope_cos, const float *rope_sin,
                              int seq, int q_heads, int k_heads, float eps, int split_half);
 
+/* The same with a second weight pair (wq_b, wk_b) for the rows from rows_a on (wq_b NULL: one pair for all rows).
+ * Calls that touch 128 MB of rows or more store with the streaming hint (iris_norm_rope_streaming_stores). */
+int iris_hip_norm_rope_hd128_streams(void *stream, uint16_t *xq, uint16_t *xk, int ld,
+                                     const float *wq, const float *wk, const float *wq_b, const float *wk_b,
+                                     int rows_a, const float *rope_cos, const float *rope_sin,
+                                     int seq, int q_heads, int k_heads, float eps, int split_half);
+int iris_norm_rope_streaming_stores(int seq, int heads_total);
+
 /* The multiplier the kernel above divides by heads_total with (0 for one head, which needs
  * none). Exported for the host-side test of the division. */
 uint32_t iris_norm_rope_magic(int heads_total);

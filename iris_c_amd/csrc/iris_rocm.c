@@ -199,6 +199,15 @@ static int aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) ==
  * work that may still read it has drained). Returns 0 after reporting a failed allocation. */
 static int scratch_fit(void **p, size_t *have, size_t need, const char *what) {
     if (need <= *have) return 1;
+    /* Growing means synchronise + free + allocate, none of which may happen while the stream is being captured into
+     * a graph (it would invalidate the capture): the call is refused with a message instead. A caller that captures a
+     * layout served through private scratch issues the call once outside the capture first; the scratch then fits. */
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(g_stream, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone) {
+        fail(-1, what, "this layout needs private scratch that has to grow, which cannot happen during stream capture: "
+                       "issue the same call once before the capture");
+        return 0;
+    }
     if (*p) {
         check(hipStreamSynchronize(g_stream), "sync");
         check(hipFree(*p), "free");
@@ -216,9 +225,10 @@ static int scratch_fit(void **p, size_t *have, size_t need, const char *what) {
 }
 
 /* Shared by the one- and two-tensor entries; xk may be NULL with k_heads 0. */
-static void norm_rope(uint16_t *xq, uint16_t *xk, int ld, const float *wq, const float *wk,
-                      const float *rope_cos, const float *rope_sin, int seq, int q_heads,
-                      int k_heads, int head_dim, float eps, int split_half) {
+static void norm_rope_streams(uint16_t *xq, uint16_t *xk, int ld, const float *wq, const float *wk,
+                              const float *wq_b, const float *wk_b, int rows_a,
+                              const float *rope_cos, const float *rope_sin, int seq, int q_heads,
+                              int k_heads, int head_dim, float eps, int split_half) {
     if (!need_ready("head_norm_rope")) return;
     if (seq <= 0 || q_heads + k_heads <= 0) return;
     if (head_dim <= 0 || (head_dim & 1) || head_dim > 1024) {
@@ -229,20 +239,34 @@ static void norm_rope(uint16_t *xq, uint16_t *xk, int ld, const float *wq, const
                aligned(rope_cos, 16) && aligned(rope_sin, 16) &&
                (long long)seq * (q_heads + k_heads) < (1 << 24) && q_heads + k_heads < 256;
     if (k_heads > 0) fast = fast && aligned(xk, 16) && aligned(wk, 16);
+    if (wq_b) fast = fast && aligned(wq_b, 16) && (k_heads == 0 || aligned(wk_b, 16));
     int err;
     if (fast) {
         g_last_kernel = "norm_rope_hd128";
-        err = iris_hip_norm_rope_hd128(g_stream, xq, xk, ld, wq, wk, rope_cos, rope_sin, seq,
-                                       q_heads, k_heads, eps, split_half != 0);
+        err = iris_hip_norm_rope_hd128_streams(g_stream, xq, xk, ld, wq, wk, wq_b, wk_b, rows_a, rope_cos, rope_sin, seq,
+                                               q_heads, k_heads, eps, split_half != 0);
     } else {
+        /* row range by row range (one when there is no second weight pair), tensor by tensor */
         g_last_kernel = "norm_rope_generic";
-        err = iris_hip_norm_rope_generic(g_stream, xq, ld, wq, rope_cos, rope_sin, seq, q_heads,
-                                         head_dim, eps, split_half != 0);
-        if (!err && k_heads > 0)
-            err = iris_hip_norm_rope_generic(g_stream, xk, ld, wk, rope_cos, rope_sin, seq,
-                                             k_heads, head_dim, eps, split_half != 0);
+        err = 0;
+        for (int part = 0; part < (wq_b ? 2 : 1) && !err; part++) {
+            const int first = part ? rows_a : 0, n = wq_b ? (part ? seq - rows_a : rows_a) : seq;
+            const float *c = rope_cos + (size_t)first * (head_dim / 2), *sn = rope_sin + (size_t)first * (head_dim / 2);
+            if (n <= 0) continue;
+            err = iris_hip_norm_rope_generic(g_stream, xq + (size_t)first * ld, ld, part ? wq_b : wq, c, sn, n, q_heads,
+                                             head_dim, eps, split_half != 0);
+            if (!err && k_heads > 0)
+                err = iris_hip_norm_rope_generic(g_stream, xk + (size_t)first * ld, ld, part ? wk_b : wk, c, sn, n,
+                                                 k_heads, head_dim, eps, split_half != 0);
+        }
     }
     if (err) check((hipError_t)err, "head_norm_rope launch");
+}
+
+static void norm_rope(uint16_t *xq, uint16_t *xk, int ld, const float *wq, const float *wk,
+                      const float *rope_cos, const float *rope_sin, int seq, int q_heads,
+                      int k_heads, int head_dim, float eps, int split_half) {
+    norm_rope_streams(xq, xk, ld, wq, wk, NULL, NULL, 0, rope_cos, rope_sin, seq, q_heads, k_heads, head_dim, eps, split_half);
 }
 
 void iris_dev_head_norm_rope(uint16_t *x, int ld, const float *w,
@@ -258,6 +282,19 @@ void iris_dev_head_norm_rope_qk(uint16_t *xq, uint16_t *xk, int ld,
                                 float eps, int split_half) {
     norm_rope(xq, xk, ld, wq, wk, rope_cos, rope_sin, seq, q_heads, k_heads, head_dim, eps,
               split_half);
+}
+
+void iris_dev_head_norm_rope_qk_streams(uint16_t *xq, uint16_t *xk, int ld,
+                                        const float *wq_a, const float *wk_a, const float *wq_b, const float *wk_b,
+                                        int rows_a, const float *rope_cos, const float *rope_sin,
+                                        int seq, int q_heads, int k_heads, int head_dim, float eps, int split_half) {
+    if (rows_a < 0 || rows_a > seq || !wq_a || !wq_b || (k_heads > 0 && (!wk_a || !wk_b || !xk))) {
+        if (need_ready("head_norm_rope_qk_streams"))
+            fail(-1, "head_norm_rope_qk_streams", "need 0 <= rows_a <= seq and both weight pairs");
+        return;
+    }
+    norm_rope_streams(xq, xk, ld, wq_a, wk_a, wq_b, wk_b, rows_a, rope_cos, rope_sin, seq, q_heads, k_heads, head_dim, eps,
+                      split_half);
 }
 
 /* wq == NULL: plain attention. Otherwise Q is normalised and rotated on the way in. */

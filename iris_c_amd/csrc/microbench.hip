@@ -90,6 +90,31 @@ __global__ void __launch_bounds__(256) k_copy(uint4 *__restrict__ dst, const uin
     }
 }
 
+/* Read-only and write-only streams, 16 B per lane, the same shape as the copy: what the memory system
+ * gives one direction alone. The sum of the read is kept alive by a store that never happens. */
+__global__ void __launch_bounds__(256) k_read_only(const uint4 *__restrict__ src, size_t n, unsigned *sink) {
+    size_t i = (size_t)blockIdx.x * 256 * 4 + threadIdx.x;
+    uint4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        size_t j = i + (size_t)u * 256;
+        v[u] = j < n ? src[j] : make_uint4(0, 0, 0, 0);
+    }
+    unsigned acc = 0;
+#pragma unroll
+    for (int u = 0; u < 4; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    if (acc == 0x9e3779b9u && n == 1) sink[0] = acc;
+}
+
+__global__ void __launch_bounds__(256) k_write_only(uint4 *__restrict__ dst, size_t n, unsigned value) {
+    size_t i = (size_t)blockIdx.x * 256 * 4 + threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        size_t j = i + (size_t)u * 256;
+        if (j < n) dst[j] = make_uint4(value, value + 1, value + 2, value + 3);
+    }
+}
+
 /* In-place read-modify-write of the same buffer (the norm+rope access pattern). */
 __global__ void __launch_bounds__(256) k_rmw(uint4 *__restrict__ buf, size_t n) {
     size_t i = (size_t)blockIdx.x * 256 * 4 + threadIdx.x;
@@ -158,6 +183,18 @@ int iris_mb_copy(void *stream, void *dst, const void *src, size_t bytes) {
     size_t n = bytes / 16;
     hipLaunchKernelGGL(k_copy, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream,
                        (uint4 *)dst, (const uint4 *)src, n);
+    return (int)hipGetLastError();
+}
+int iris_mb_read(void *stream, const void *src, size_t bytes, void *sink) {
+    size_t n = bytes / 16;
+    hipLaunchKernelGGL(k_read_only, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint4 *)src, n, (unsigned *)sink);
+    return (int)hipGetLastError();
+}
+int iris_mb_write(void *stream, void *dst, size_t bytes) {
+    size_t n = bytes / 16;
+    hipLaunchKernelGGL(k_write_only, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream,
+                       (uint4 *)dst, n, 7u);
     return (int)hipGetLastError();
 }
 int iris_mb_rmw(void *stream, void *buf, size_t bytes) {

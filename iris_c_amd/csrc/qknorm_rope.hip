@@ -35,12 +35,20 @@ constexpr int kThreads = 256;
 constexpr int kUnroll = 2;                       /* vectors in flight per 16-lane row */
 constexpr int kUnitsPerBlock = (kThreads / 16) * kUnroll;
 
-template <bool SPLIT>
+/* A second weight pair for the rows from `rows_a` on (STREAMS): the double-stream block normalises the text rows
+ * and the image rows of the joint q | k | v buffer with different weights (reference
+ * iris_transformer_flux.c:3796-3803, four calls); here they are one launch over all rows. */
+struct SecondStream {
+    const float *wq, *wk;
+    int first_unit;                               /* rows_a * heads_total */
+};
+
+template <bool SPLIT, bool STREAMS, bool STREAMING_STORES>
 __global__ void __launch_bounds__(kThreads)
 k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
                   const float *__restrict__ wq, const float *__restrict__ wk,
                   const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
-                  int units, int q_heads, int heads_total, uint32_t magic, float eps) {
+                  int units, int q_heads, int heads_total, uint32_t magic, float eps, SecondStream second) {
     const int sub = threadIdx.x & 15;             /* which 16 B of the 256 B vector */
     const int row = threadIdx.x >> 4;             /* 16-lane row inside the block */
     const int first = blockIdx.x * kUnitsPerBlock + row;
@@ -56,12 +64,13 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
     u32x4 raw[kUnroll];
     float4 ct[kUnroll][TN], st[kUnroll][TN];
     uint16_t *ptr[kUnroll];
-    bool isk[kUnroll];
+    bool isk[kUnroll], later[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
         int unit = first + u * (kThreads / 16);
         const bool live = unit < units;
         unit = live ? unit : 0;
+        later[u] = STREAMS && unit >= second.first_unit;
         /* unit / heads_total; one head per token has no 32-bit magic (it would be 2^32) */
         const int s = heads_total == 1 ? unit : (int)__umulhi((uint32_t)unit, magic);
         const int h = unit - s * heads_total;
@@ -88,6 +97,16 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
         wq8[0] = a0.x; wq8[1] = a0.y; wq8[2] = a0.z; wq8[3] = a0.w; wq8[4] = a1.x; wq8[5] = a1.y; wq8[6] = a1.z; wq8[7] = a1.w;
         wk8[0] = b0.x; wk8[1] = b0.y; wk8[2] = b0.z; wk8[3] = b0.w; wk8[4] = b1.x; wk8[5] = b1.y; wk8[6] = b1.z; wk8[7] = b1.w;
     }
+    float wq8b[8], wk8b[8];                         /* the second stream's pair */
+    if (STREAMS) {
+        const float4 a0 = *reinterpret_cast<const float4 *>(second.wq + sub * 8);
+        const float4 a1 = *reinterpret_cast<const float4 *>(second.wq + sub * 8 + 4);
+        const float *wks = heads_total > q_heads ? second.wk : second.wq;
+        const float4 b0 = *reinterpret_cast<const float4 *>(wks + sub * 8);
+        const float4 b1 = *reinterpret_cast<const float4 *>(wks + sub * 8 + 4);
+        wq8b[0] = a0.x; wq8b[1] = a0.y; wq8b[2] = a0.z; wq8b[3] = a0.w; wq8b[4] = a1.x; wq8b[5] = a1.y; wq8b[6] = a1.z; wq8b[7] = a1.w;
+        wk8b[0] = b0.x; wk8b[1] = b0.y; wk8b[2] = b0.z; wk8b[3] = b0.w; wk8b[4] = b1.x; wk8b[5] = b1.y; wk8b[6] = b1.z; wk8b[7] = b1.w;
+    }
 
     /* Phase 2: normalise, rotate, store. */
 #pragma unroll
@@ -100,13 +119,20 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
         sv[4] = st[u][TN - 1].x; sv[5] = st[u][TN - 1].y; sv[6] = st[u][TN - 1].z; sv[7] = st[u][TN - 1].w;
         float w8[8];
 #pragma unroll
-        for (int i = 0; i < 8; i++) w8[i] = isk[u] ? wk8[i] : wq8[i];
+        for (int i = 0; i < 8; i++) {
+            w8[i] = isk[u] ? wk8[i] : wq8[i];
+            if (STREAMS) w8[i] = later[u] ? (isk[u] ? wk8b[i] : wq8b[i]) : w8[i];
+        }
         const u32x4 out = nr_vector_hd128<SPLIT>(raw[u], w8, cv, sv, eps, sub);
         /* Write-through store (sc0 sc1): the rows leave the L2 as they are produced instead of at the
          * end-of-kernel write-back, 2-5 % faster on 59-118 MB calls whether the rows were cached or not.
-         * (Adding the streaming hint `nt` takes the two-tensor call on uncached rows from 23.0 to 21.2 us
-         * but a call on rows that sit in the Infinity Cache from 9.4 to 12.7 us: not taken.) */
-        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" :: "v"(ptr[u]), "v"(out) : "memory");
+         * Adding the streaming hint `nt` takes the two-tensor call on uncached rows from 23.0 to 21.2 us
+         * but a call on rows that sit in the Infinity Cache from 9.4 to 12.7 us: it is taken
+         * (STREAMING_STORES) only by calls so large that their rows cannot be resident in that cache. */
+        if (STREAMING_STORES)
+            asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" :: "v"(ptr[u]), "v"(out) : "memory");
+        else
+            asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" :: "v"(ptr[u]), "v"(out) : "memory");
     }
 }
 
@@ -145,24 +171,61 @@ extern "C" uint32_t iris_norm_rope_magic(int heads_total) {
     return (uint32_t)((0x100000000ull + (uint64_t)heads_total - 1) / (uint64_t)heads_total);
 }
 
-extern "C" int iris_hip_norm_rope_hd128(void *stream, uint16_t *xq, uint16_t *xk, int ld,
-                                        const float *wq, const float *wk,
-                                        const float *rope_cos, const float *rope_sin,
-                                        int seq, int q_heads, int k_heads, float eps,
-                                        int split_half) {
+/* Rows that a call touches, from which size on they cannot all be resident in the 256 MB Infinity Cache together
+ * with what else a model keeps there: such calls store with the streaming hint. */
+static const long long kStreamingStoreBytes = 128ll << 20;
+
+extern "C" int iris_norm_rope_streaming_stores(int seq, int heads_total) {
+    return (long long)seq * heads_total * 256 >= kStreamingStoreBytes;
+}
+
+template <bool SPLIT, bool STREAMS>
+static int launch_norm_rope(hipStream_t st, int blocks, bool streaming, uint16_t *xq, uint16_t *xk, int ld, const float *wq,
+                            const float *wk, const float *rope_cos, const float *rope_sin, int units, int q_heads,
+                            int heads_total, uint32_t magic, float eps, SecondStream second) {
+    if (streaming)
+        hipLaunchKernelGGL((k_norm_rope_hd128<SPLIT, STREAMS, true>), dim3(blocks), dim3(kThreads), 0, st, xq, xk, ld,
+                           wq, wk, rope_cos, rope_sin, units, q_heads, heads_total, magic, eps, second);
+    else
+        hipLaunchKernelGGL((k_norm_rope_hd128<SPLIT, STREAMS, false>), dim3(blocks), dim3(kThreads), 0, st, xq, xk, ld,
+                           wq, wk, rope_cos, rope_sin, units, q_heads, heads_total, magic, eps, second);
+    return (int)hipGetLastError();
+}
+
+/* wq_b == NULL: one weight pair for all rows. Otherwise rows [rows_a, seq) take (wq_b, wk_b). */
+extern "C" int iris_hip_norm_rope_hd128_streams(void *stream, uint16_t *xq, uint16_t *xk, int ld,
+                                                const float *wq, const float *wk, const float *wq_b, const float *wk_b,
+                                                int rows_a, const float *rope_cos, const float *rope_sin,
+                                                int seq, int q_heads, int k_heads, float eps, int split_half) {
     const int heads_total = q_heads + k_heads;
     const int units = seq * heads_total;
     if (units <= 0) return 0;
     const uint32_t magic = iris_norm_rope_magic(heads_total);
     const int blocks = (units + kUnitsPerBlock - 1) / kUnitsPerBlock;
     hipStream_t st = (hipStream_t)stream;
+    const bool streaming = iris_norm_rope_streaming_stores(seq, heads_total) != 0;
+    const SecondStream second = {wq_b, wk_b, rows_a * heads_total};
+    if (wq_b) {
+        if (split_half)
+            return launch_norm_rope<true, true>(st, blocks, streaming, xq, xk, ld, wq, wk, rope_cos, rope_sin, units, q_heads,
+                                                heads_total, magic, eps, second);
+        return launch_norm_rope<false, true>(st, blocks, streaming, xq, xk, ld, wq, wk, rope_cos, rope_sin, units, q_heads,
+                                             heads_total, magic, eps, second);
+    }
     if (split_half)
-        hipLaunchKernelGGL(k_norm_rope_hd128<true>, dim3(blocks), dim3(kThreads), 0, st, xq, xk, ld,
-                           wq, wk, rope_cos, rope_sin, units, q_heads, heads_total, magic, eps);
-    else
-        hipLaunchKernelGGL(k_norm_rope_hd128<false>, dim3(blocks), dim3(kThreads), 0, st, xq, xk, ld,
-                           wq, wk, rope_cos, rope_sin, units, q_heads, heads_total, magic, eps);
-    return (int)hipGetLastError();
+        return launch_norm_rope<true, false>(st, blocks, streaming, xq, xk, ld, wq, wk, rope_cos, rope_sin, units, q_heads,
+                                             heads_total, magic, eps, second);
+    return launch_norm_rope<false, false>(st, blocks, streaming, xq, xk, ld, wq, wk, rope_cos, rope_sin, units, q_heads,
+                                          heads_total, magic, eps, second);
+}
+
+extern "C" int iris_hip_norm_rope_hd128(void *stream, uint16_t *xq, uint16_t *xk, int ld,
+                                        const float *wq, const float *wk,
+                                        const float *rope_cos, const float *rope_sin,
+                                        int seq, int q_heads, int k_heads, float eps,
+                                        int split_half) {
+    return iris_hip_norm_rope_hd128_streams(stream, xq, xk, ld, wq, wk, nullptr, nullptr, 0, rope_cos, rope_sin, seq,
+                                            q_heads, k_heads, eps, split_half);
 }
 
 extern "C" int iris_hip_norm_rope_generic(void *stream, uint16_t *x, int ld, const float *w,

@@ -105,6 +105,40 @@ def main():
     out = os.path.join(HERE, "ref_vectors.npz")
     np.savez_compressed(out, **g)
     print("wrote", out, os.path.getsize(out), "bytes,", len(g), "arrays")
+    c1_chain(ref, refi)
+
+
+C1_ROWS = [0, 1, 17, 31, 32, 63, 64, 65, 79, 80, 127, 128, 159, 191, 192, 200, 255, 256, 257, 300, 318, 319]
+
+
+def c1_chain(ref, refi):
+    """The metric's own chain at head_dim 128, configuration C1 at full shape (24 heads x 128, 64 text + 16 x 16
+    image tokens), through the reference's compiled code: apply_qk_norm -> apply_rope_2d on Q and on K ->
+    iris_flash_attention (iris_transformer_flux.c:1289-1343, 952-974, iris_kernels.c:899-991). The inputs are the
+    seeded draws of tests/workloads.py:c1 (generator bit-exact with the reference's, checked here), rounded to bf16 and
+    taken as f32; the tables are the reference's own full [seq, 128] tables. Stored: the reference's Q and K after
+    norm + rope and its attention output, on C1_ROWS (both streams, both sides of the text / image boundary)."""
+    import workloads as W
+    case = W.c1()
+    seq, heads, hd, dim = case["seq"], 24, 128, 3072
+    st_check = R.randn(refi, W.SEED0 + 1, 512)
+    orc = oracle.oracle()
+    assert np.array_equal(st_check.view(np.uint32), orc.randn(orc.rng(W.SEED0 + 1), 512).view(np.uint32))
+    f = oracle.bf16_to_f32(case["buf"])
+    q, k, v = (np.ascontiguousarray(f[:, i * dim:(i + 1) * dim]) for i in range(3))
+    ct, st = R.flux2_rope_text(refi, 64)
+    ci, si = R.flux2_rope_2d(refi, 16, 16)
+    cos_full, sin_full = np.concatenate([ct, ci]), np.concatenate([st, si])
+    assert np.array_equal(np.ascontiguousarray(cos_full[:, 0::2]).view(np.uint32), case["cos"].view(np.uint32))
+    qn, kn = R.flux2_qk_norm(ref, q.reshape(seq, heads, hd), k.reshape(seq, heads, hd), case["wq"], case["wk"], case["eps"])
+    qr = R.flux2_apply_rope_2d(ref, qn, cos_full, sin_full).reshape(seq, dim)
+    kr = R.flux2_apply_rope_2d(ref, kn, cos_full, sin_full).reshape(seq, dim)
+    o = R.attention_flash(ref, qr, kr, v, heads, case["scale"])
+    rows = np.array(C1_ROWS)
+    out = os.path.join(HERE, "c1_chain.npz")
+    np.savez_compressed(out, rows=rows, q_rows=qr[rows], k_rows=kr[rows], out_rows=o[rows],
+                        out_checksum=np.array([np.float64(o.astype(np.float64).sum()), np.float64(np.abs(o).astype(np.float64).sum())]))
+    print("wrote", out, os.path.getsize(out), "bytes")
 
 
 if __name__ == "__main__":

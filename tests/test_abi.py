@@ -109,7 +109,8 @@ def test_path_only_archive_links_next_to_a_host_backend():
     out = subprocess.run(["nm", "--defined-only", os.path.join(ROOT, "iris_c_amd", "libiris_dev_path.a")],
                          capture_output=True, text=True, check=True).stdout
     defined = {line.split()[-1] for line in out.splitlines() if " T iris_dev_" in line}
-    assert defined == {"iris_dev_head_norm_rope", "iris_dev_head_norm_rope_qk", "iris_dev_attention", "iris_dev_attention_qnorm",
+    assert defined == {"iris_dev_head_norm_rope", "iris_dev_head_norm_rope_qk", "iris_dev_head_norm_rope_qk_streams", "iris_dev_attention",
+                       "iris_dev_attention_qnorm",
                        "iris_dev_last_error", "iris_dev_last_kernel", "iris_dev_path_attach", "iris_dev_path_detach"}
     text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "iris_dev_path.h")).read(), flags=re.S)
     assert set(re.findall(r"\b(iris_dev_\w+)\s*\(", text)) == {"iris_dev_path_attach", "iris_dev_path_detach"}

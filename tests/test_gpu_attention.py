@@ -63,6 +63,26 @@ def test_c1_plumbing_full_size(dev, orc, fa):
     assert_close(got, flash, "C1 vs flash")
 
 
+def test_c1_against_the_vector_the_compiled_reference_wrote(dev, fa):
+    """C1 at full shape (24 x 128, 64 text + 256 image tokens): norm + rope on Q and K, then attention, on the GPU,
+    against the output rows that the reference's own compiled apply_qk_norm -> apply_rope_2d ->
+    iris_flash_attention produced from the same seeded inputs (tests/golden/c1_chain.npz, written by
+    tests/golden/make_golden.py where the reference tree is present). The stated bar of the bf16 path."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "c1_chain.npz"), allow_pickle=False)
+    case = after_norm_rope(dev, W.c1())
+    got, kernel = gpu_attention(dev, case)
+    assert kernel == fa
+    assert_close(got[g["rows"]], g["out_rows"], "C1 vs the reference's vector")
+    # the same with Q normalised inside the attention kernel
+    raw = W.c1()
+    buf = dev.norm_rope(raw["buf"], raw["ldi"], 3072, raw["wk"], raw["cos"], raw["sin"], raw["seq"], 24, 128, raw["eps"], 0)
+    out, kernel, _ = dev.attention_qnorm(buf, raw["ldi"], 0, 3072, 6144, raw["seq"], raw["seq"], 24, 24, 128, raw["scale"],
+                                         raw["wq"], raw["cos"], raw["sin"], raw["eps"], 0)
+    assert kernel == "fa_hd128_qnorm"
+    assert_close(O.bf16_to_f32(out)[g["rows"]], g["out_rows"], "C1 (Q norm inside attention) vs the reference's vector")
+
+
 @pytest.mark.parametrize("maker,shrink", [(W.c2, 8), (W.c5, 32)])
 def test_joint_attention_shrunk(dev, orc, fa, maker, shrink):
     case = after_norm_rope(dev, maker(shrink))

@@ -235,3 +235,214 @@ def test_vae_resblock_and_attention_chain(dev, orc):
     assert mx <= 3e-2 and mean <= 3e-3, f"resblock: max-abs {mx:.4g}, mean-abs {mean:.4g}"
     mx, mean = error_stats(got_att - xa, want_att - xa)
     assert mx <= 3e-2 and mean <= 3e-3, f"attention block: max-abs {mx:.4g}, mean-abs {mean:.4g}"
+
+
+# ------------------------------------------------------------------ double-stream (MM-DiT) block (iris_transformer_flux.c:3786-3823)
+def make_double_block(seed, txt, img, heads, mlp):
+    """Two streams, text rows [0, txt) and image rows [txt, txt + img), each with its own modulation, projections and
+    Q / K norm weights; one rotary table over the joint sequence."""
+    rng = np.random.default_rng(seed)
+    dim, seq = heads * 128, txt + img
+    f = lambda *shape, s=1.0: (rng.standard_normal(shape, dtype=np.float32) * np.float32(s))
+    ang = rng.uniform(-3.0, 3.0, (seq, 64)).astype(np.float32)
+    streams = []
+    for _ in range(2):
+        streams.append(dict(mod=f(6 * dim, s=0.3), qkv=O.f32_to_bf16(f(3 * dim, dim, s=1.0 / np.sqrt(dim))),
+                            proj=O.f32_to_bf16(f(dim, dim, s=1.0 / np.sqrt(dim))),
+                            norm_q=1 + f(128, s=0.05), norm_k=1 + f(128, s=0.05),
+                            ff_in=O.f32_to_bf16(f(2 * mlp, dim, s=1.0 / np.sqrt(dim))) if mlp else None,
+                            ff_out=O.f32_to_bf16(f(dim, mlp, s=1.0 / np.sqrt(mlp))) if mlp else None))
+    return dict(txt=txt, img=img, seq=seq, heads=heads, dim=dim, mlp=mlp, x=f(seq, dim, s=1.5) + np.float32(0.2), streams=streams,
+                cos=np.cos(ang), sin=np.sin(ang), scale=float(1.0 / np.sqrt(128.0)))
+
+
+def stream_rows(b):
+    return ((0, b["txt"]), (b["txt"], b["img"]))
+
+
+def device_double_block(dev, b, fused_qk=False, snapshots=False):
+    """The calls of the reference's loop body, in its order and with its pointers: per stream the q | k | v rows at
+    h + 3 first dim, the tables at rope + first 64, that stream's norm weights; one attention over all rows; per stream
+    the output projection and the gated residual; then the two feed-forward halves. With `snapshots` the q | k | v rows
+    are downloaded before and after the norm calls and the attention output after the attention call."""
+    lib = dev.lib
+    seq, dim, mlp, heads = b["seq"], b["dim"], b["mlp"], b["heads"]
+    x = dev.put(b["x"])
+    cos, sin = dev.put(b["cos"]), dev.put(b["sin"])
+    ds = [{k: dev.put(v) for k, v in s.items() if v is not None} for s in b["streams"]]
+    norm = dev.alloc(seq * dim * 2)
+    h = dev.alloc(seq * max(3 * dim, 2 * mlp) * 2)
+    cat = dev.alloc(seq * max(dim, mlp) * 2)
+    out = dev.alloc(seq * dim * 4)
+    snap = {}
+    for m, (first, n) in enumerate(stream_rows(b)):
+        s = ds[m]
+        qkv = ptr_add(h, 2 * 3 * first * dim)
+        lib.iris_dev_layer_norm_mod(norm, ptr_add(x, 4 * first * dim), s["mod"], ptr_add(s["mod"], 4 * dim), n, dim, 1e-6)
+        lib.iris_dev_linear_bf16(qkv, norm, s["qkv"], n, dim, 3 * dim)
+    if snapshots:
+        dev.check()
+        snap["h_before"] = dev.get(h, (seq, 3 * dim), np.uint16)
+    kernels = []
+    if fused_qk == "streams":                        # the four calls as one launch over the joint rows
+        lib.iris_dev_head_norm_rope_qk_streams(h, ptr_add(h, 2 * dim), 3 * dim, ds[0]["norm_q"], ds[0]["norm_k"], ds[1]["norm_q"],
+                                               ds[1]["norm_k"], b["txt"], cos, sin, seq, heads, heads, 128, 1e-6, 0)
+        kernels += [dev.dev.last_kernel()] * 2
+    for m, (first, n) in enumerate(stream_rows(b)):
+        if fused_qk == "streams":
+            break
+        s = ds[m]
+        qkv = ptr_add(h, 2 * 3 * first * dim)
+        rc, rs = ptr_add(cos, 4 * first * 64), ptr_add(sin, 4 * first * 64)
+        if fused_qk:
+            lib.iris_dev_head_norm_rope_qk(qkv, ptr_add(qkv, 2 * dim), 3 * dim, s["norm_q"], s["norm_k"], rc, rs, n, heads, heads,
+                                           128, 1e-6, 0)
+        else:
+            lib.iris_dev_head_norm_rope(qkv, 3 * dim, s["norm_q"], rc, rs, n, heads, 128, 1e-6, 0)
+            lib.iris_dev_head_norm_rope(ptr_add(qkv, 2 * dim), 3 * dim, s["norm_k"], rc, rs, n, heads, 128, 1e-6, 0)
+        kernels.append(dev.dev.last_kernel())
+    if snapshots:
+        dev.check()
+        snap["h_after"] = dev.get(h, (seq, 3 * dim), np.uint16)
+    lib.iris_dev_attention(cat, dim, h, ptr_add(h, 2 * dim), ptr_add(h, 4 * dim), 3 * dim, seq, seq, heads, heads, 128, b["scale"], 0, None)
+    kernels.append(dev.dev.last_kernel())
+    if snapshots:
+        dev.check()
+        snap["cat"] = dev.get(cat, (seq, dim), np.uint16)
+    for m, (first, n) in enumerate(stream_rows(b)):
+        s = ds[m]
+        lib.iris_dev_linear_f32(out, ptr_add(cat, 2 * first * dim), s["proj"], n, dim, dim)
+        lib.iris_dev_residual(ptr_add(x, 4 * first * dim), out, ptr_add(s["mod"], 4 * 2 * dim), n, dim)
+    if snapshots:
+        dev.check()
+        snap["x_mid"] = dev.get(x, (seq, dim), np.float32)
+    if mlp:
+        for m, (first, n) in enumerate(stream_rows(b)):
+            s = ds[m]
+            xs = ptr_add(x, 4 * first * dim)
+            lib.iris_dev_layer_norm_mod(norm, xs, ptr_add(s["mod"], 4 * 3 * dim), ptr_add(s["mod"], 4 * 4 * dim), n, dim, 1e-6)
+            lib.iris_dev_linear_bf16(h, norm, s["ff_in"], n, dim, 2 * mlp)
+            lib.iris_dev_swiglu(cat, mlp, h, ptr_add(h, 2 * mlp), 2 * mlp, n, mlp)
+            lib.iris_dev_linear_f32(out, cat, s["ff_out"], n, mlp, dim)
+            lib.iris_dev_residual(xs, out, ptr_add(s["mod"], 4 * 5 * dim), n, dim)
+    dev.check()
+    got = dev.get(x, (seq, dim), np.float32)
+    dev.free_all()
+    return got, kernels, snap
+
+
+def oracle_double_block(orc, b):
+    seq, dim, mlp, heads = b["seq"], b["dim"], b["mlp"], b["heads"]
+    x = b["x"].copy()
+    h = np.zeros((seq, 3 * dim), np.uint16)
+    for m, (first, n) in enumerate(stream_rows(b)):
+        s = b["streams"][m]
+        norm = orc.dev_layer_norm_mod(np.ascontiguousarray(x[first:first + n]), s["mod"][:dim], s["mod"][dim:2 * dim], 1e-6)
+        h[first:first + n] = O.f32_to_bf16(orc.dev_linear(norm, s["qkv"]))
+        rc, rs = b["cos"][first:first + n], b["sin"][first:first + n]
+        orc.head_norm_rope_bf16(h, 3 * dim, s["norm_q"], rc, rs, n, heads, 128, 1e-6, 0, col0=first * 3 * dim)
+        orc.head_norm_rope_bf16(h, 3 * dim, s["norm_k"], rc, rs, n, heads, 128, 1e-6, 0, col0=first * 3 * dim + dim)
+    cat = O.f32_to_bf16(orc.attention_bf16(h, 3 * dim, 0, dim, 2 * dim, seq, seq, heads, heads, 128, b["scale"]))
+    for m, (first, n) in enumerate(stream_rows(b)):
+        s = b["streams"][m]
+        out = orc.dev_linear(np.ascontiguousarray(cat[first:first + n]), s["proj"])
+        x[first:first + n] = orc.dev_residual(np.ascontiguousarray(x[first:first + n]), out, s["mod"][2 * dim:3 * dim])
+    x_mid = x.copy()
+    if mlp:
+        for m, (first, n) in enumerate(stream_rows(b)):
+            s = b["streams"][m]
+            xs = np.ascontiguousarray(x[first:first + n])
+            norm = orc.dev_layer_norm_mod(xs, s["mod"][3 * dim:4 * dim], s["mod"][4 * dim:5 * dim], 1e-6)
+            act = orc.dev_swiglu(O.f32_to_bf16(orc.dev_linear(norm, s["ff_in"])), mlp)
+            x[first:first + n] = orc.dev_residual(xs, orc.dev_linear(act, s["ff_out"]), s["mod"][5 * dim:6 * dim])
+    return x, x_mid
+
+
+@pytest.mark.parametrize("txt,img,heads,mlp,backend", [(48, 272, 3, 768, 1), (37, 219, 2, 512, 0), (300, 724, 2, 0, 1)])
+def test_double_stream_block_chain(dev, orc, txt, img, heads, mlp, backend):
+    """The double-stream block as the reference issues it: FOUR norm+rope launches on row sub-ranges of the joint
+    q | k | v rows (text rows, image rows; Q and K each) with the stream's own weight pair and the tables offset to the
+    stream's first row, then one attention over all rows, then per stream projection + gated residual and the
+    feed-forward half. Compared in full with the same chain composed from the oracle."""
+    b = make_double_block(100 + txt, txt, img, heads, mlp)
+    dev.lib.iris_dev_linear_backend(backend)
+    try:
+        got, kernels, _ = device_double_block(dev, b)
+        fused, kernels_fused, _ = device_double_block(dev, b, fused_qk=True)
+    finally:
+        dev.lib.iris_dev_linear_backend(0)
+    assert kernels == ["norm_rope_hd128", "norm_rope_hd128", "fa_hd128"], kernels
+    want, _ = oracle_double_block(orc, b)
+    mx, mean = error_stats(got - b["x"], want - b["x"])
+    assert mx <= 3e-2 and mean <= 3e-3, f"max-abs {mx:.4g}, mean-abs {mean:.4g}"
+    upd = np.abs(want - b["x"])
+    assert mean <= 0.01 * upd.mean(), f"mean-abs {mean:.4g} against a mean update of {upd.mean():.4g}"
+    # both streams moved, and by different amounts (their weights differ): a chain that used one stream's weights for
+    # both, or the tables from row 0 for the image rows, fails the comparison above; this guards the test data
+    assert upd[:txt].mean() > 0.02 and upd[txt:].mean() > 0.02
+    assert np.array_equal(got, fused), "one Q+K launch per stream differs from the four calls"
+    dev.lib.iris_dev_linear_backend(backend)
+    try:
+        one, kernels_one, _ = device_double_block(dev, b, fused_qk="streams")
+    finally:
+        dev.lib.iris_dev_linear_backend(0)
+    assert kernels_one == kernels
+    assert np.array_equal(got, one), "one launch for both streams differs from the four calls"
+
+
+def test_double_stream_block_full_size(dev, orc):
+    """The same block at the benchmark configuration's size (512 text + 4096 image rows, 24 heads, width 3072; its
+    attention half). The four norm+rope launches are compared with the oracle on EVERY row (from the device's own
+    projection output); the projection, the attention output and the residual update on sampled rows of both streams,
+    the stream boundary among them."""
+    b = make_double_block(7, 512, 4096, 24, 0)
+    seq, dim, heads, txt = b["seq"], b["dim"], b["heads"], b["txt"]
+    dev.lib.iris_dev_linear_backend(1)
+    try:
+        got, kernels, snap = device_double_block(dev, b, snapshots=True)
+    finally:
+        dev.lib.iris_dev_linear_backend(0)
+    assert kernels == ["norm_rope_hd128", "norm_rope_hd128", "fa_hd128"], kernels
+    rows = np.array(sorted(set([0, 1, 255, 510, 511, 512, 513, 767, 2047, 2048, 3000, 4095, 4096, 4351, 4606, 4607])))
+    # 1. projection on sampled rows
+    for m, (first, n) in enumerate(stream_rows(b)):
+        s = b["streams"][m]
+        mine = rows[(rows >= first) & (rows < first + n)]
+        norm = orc.dev_layer_norm_mod(np.ascontiguousarray(b["x"][mine]), s["mod"][:dim], s["mod"][dim:2 * dim], 1e-6)
+        want = orc.dev_linear(norm, s["qkv"])
+        mx, mean = error_stats(O.bf16_to_f32(snap["h_before"][mine]), want)
+        assert mx <= 3e-2 and mean <= 3e-3, f"projection, stream {m}: max-abs {mx:.4g}, mean-abs {mean:.4g}"
+    # 2. the four norm+rope launches, all rows, Q and K columns; V columns untouched
+    want_h = snap["h_before"].copy()
+    for m, (first, n) in enumerate(stream_rows(b)):
+        s = b["streams"][m]
+        rc, rs = b["cos"][first:first + n], b["sin"][first:first + n]
+        orc.head_norm_rope_bf16(want_h, 3 * dim, s["norm_q"], rc, rs, n, heads, 128, 1e-6, 0, col0=first * 3 * dim)
+        orc.head_norm_rope_bf16(want_h, 3 * dim, s["norm_k"], rc, rs, n, heads, 128, 1e-6, 0, col0=first * 3 * dim + dim)
+    assert np.array_equal(snap["h_after"][:, 2 * dim:], snap["h_before"][:, 2 * dim:]), "V columns changed"
+    g, w = O.bf16_to_f32(snap["h_after"][:, :2 * dim]), O.bf16_to_f32(want_h[:, :2 * dim])
+    ulp = np.maximum(np.abs(w), 2.0 ** -126) * 2.0 ** -7          # one bf16 step at the expected value
+    worst = np.abs(g - w) / ulp
+    assert worst.max() <= 1.0 + 1e-6 or np.abs(g - w).max() <= 1e-5, f"norm+rope off by {worst.max():.3g} bf16 steps"
+    assert (snap["h_after"][:, :2 * dim] != want_h[:, :2 * dim]).mean() < 0.02, "more than 2 % of the entries differ in the last bit"
+    # 3. attention on sampled rows, from the device's normalised rows
+    want_att = orc.attention_bf16(snap["h_after"], 3 * dim, 0, dim, 2 * dim, seq, seq, heads, heads, 128, b["scale"], rows=rows)
+    from gpu_harness import assert_parity
+    assert_parity(O.bf16_to_f32(snap["cat"][rows]), want_att, "attention of the joint block")
+    # 4. projection + gated residual on sampled rows, from the device's attention output
+    for m, (first, n) in enumerate(stream_rows(b)):
+        s = b["streams"][m]
+        mine = rows[(rows >= first) & (rows < first + n)]
+        out = orc.dev_linear(np.ascontiguousarray(snap["cat"][mine]), s["proj"])
+        want = orc.dev_residual(np.ascontiguousarray(b["x"][mine]), out, s["mod"][2 * dim:3 * dim])
+        mx, mean = error_stats(got[mine] - b["x"][mine], want - b["x"][mine])
+        assert mx <= 3e-2 and mean <= 3e-3, f"residual update, stream {m}: max-abs {mx:.4g}, mean-abs {mean:.4g}"
+    assert np.array_equal(got, snap["x_mid"])
+    # the one-launch form of the four norm calls: same rows, bit for bit
+    dev.lib.iris_dev_linear_backend(1)
+    try:
+        _, _, snap_one = device_double_block(dev, b, fused_qk="streams", snapshots=True)
+    finally:
+        dev.lib.iris_dev_linear_backend(0)
+    assert np.array_equal(snap_one["h_before"], snap["h_before"])
+    assert np.array_equal(snap_one["h_after"], snap["h_after"]), "one launch for both streams differs from the four calls"

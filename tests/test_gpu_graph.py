@@ -1,5 +1,6 @@
 """The hot path under HIP graph capture. The library enqueues on one stream that it hands out
-(iris_dev_stream), and the two hot-path operators allocate nothing, so a caller can capture a
+(iris_dev_stream), and the two hot-path operators allocate nothing on the layouts the matrix-core
+kernels take directly (head_dim 128 / 256 / 512, 16-byte aligned rows), so a caller can capture a
 step -- norm+rope on Q, on K, attention -- into a graph once and replay it (what a launch-bound loop
 such as the 36 layers of the text encoder wants). Every replay is checked against the eager result,
 with eager work and synchronisations of the program between the replays.
@@ -70,5 +71,44 @@ def test_step_replayed_from_a_graph_equals_the_eager_step(maker):
         dev.check()
         got = dev.get(out, (seq, case["ldo"]), np.uint16)
         assert np.array_equal(got, want), f"replay {replay} differs from the eager step"
+    g.rt.hipGraphExecDestroy(run)
+    dev.free_all()
+
+
+def test_a_layout_that_needs_scratch_is_refused_during_capture_until_the_scratch_exists():
+    """head_dim 64 runs on the matrix cores through a padded private copy of q | k | v. Growing that copy means
+    synchronise + free + allocate, which would invalidate a capture: inside a capture the call is refused (error
+    reported, nothing enqueued, the capture stays valid); after one call outside, the same call is captured and
+    replays to the eager result."""
+    import oracle as O
+    dev, g = Dev(), Graphs()
+    lib, stream = dev.lib, _vp(dev.lib.iris_dev_stream())
+    rng = np.random.default_rng(3)
+    seq, heads, hd = 30000, 2, 64          # a 46 MB copy: larger than anything another test has left in the scratch
+    buf = O.f32_to_bf16(rng.standard_normal((seq, 3 * heads * hd)).astype(np.float32))
+    rows, out = dev.put(buf), dev.alloc(seq * heads * hd * 2)
+    args = (out, heads * hd, rows, ptr_add(rows, 2 * heads * hd), ptr_add(rows, 4 * heads * hd), 3 * heads * hd, seq, seq, heads, heads, hd,
+            0.125, 0, None)
+    assert g.rt.hipStreamBeginCapture(stream, 0) == 0
+    lib.iris_dev_attention(*args)
+    refused = lib.iris_dev_last_error()
+    graph = _vp()
+    assert g.rt.hipStreamEndCapture(stream, C.byref(graph)) == 0, "the refused call must leave the capture valid"
+    if graph:
+        g.rt.hipGraphDestroy(graph)
+    assert refused == -1
+    lib.iris_dev_attention(*args)                                   # outside: allocates the scratch
+    dev.check()
+    assert dev.dev.last_kernel() == "fa_hd128_packed"
+    want = dev.get(out, (seq, heads * hd), np.uint16)
+    assert want.any()
+    run = g.capture(stream, lambda: lib.iris_dev_attention(*args))
+    dev.check()
+    for replay in range(2):
+        junk = np.full((seq, heads * hd), 0x7fc0 + replay, np.uint16)
+        lib.iris_dev_upload(out, junk.ctypes.data_as(_vp), junk.nbytes)
+        assert g.rt.hipGraphLaunch(run, stream) == 0
+        lib.iris_dev_sync()
+        assert np.array_equal(dev.get(out, (seq, heads * hd), np.uint16), want)
     g.rt.hipGraphExecDestroy(run)
     dev.free_all()

@@ -72,6 +72,39 @@ def test_linear(dev, orc, rows, k, out, out_bf16, backend):
         assert np.abs(got - want).max() <= scale * 2e-5
 
 
+@pytest.mark.parametrize("rows,k,out,width", [(4608, 128, 9216, 224), (4608, 256, 3072, 224), (4608, 128, 27648, 256), (2048, 128, 2048, 192)])
+@pytest.mark.parametrize("out_bf16", [False, True])
+def test_four_wave_gemm_every_tile_width(dev, orc, rows, k, out, width, out_bf16):
+    """The four-wave kernel at each of its tile widths (192, 224, 256 columns), f32 and bf16 output, WHOLE output:
+    the widths the model projections take (4608 rows -> 9216 / 3072 columns: 224, with a last tile moved back because
+    9216 % 224 != 0; -> 27648: 256) with a short reduction so that the comparison stays cheap. Against a float64
+    product of the same bf16 operands (numpy's BLAS, an independent routine; the f32 accumulation error over 128-256
+    terms is far below the bar), and the oracle on sampled rows."""
+    import ctypes as C
+    plan = (C.c_int * 2)()
+    dev.lib.iris_hip_linear_plan(rows, k, out, 2 if out_bf16 else 4, plan)
+    assert (plan[0], plan[1]) == (3, width), list(plan)
+    x, W = O.f32_to_bf16(rnd((rows, k), rows + k)), O.f32_to_bf16(rnd((out, k), out, 0.05))
+    want = O.bf16_to_f32(x).astype(np.float64) @ O.bf16_to_f32(W).astype(np.float64).T
+    pick = np.random.default_rng(out).integers(0, rows, 16)
+    np.testing.assert_allclose(orc.dev_linear(np.ascontiguousarray(x[pick]), W), want[pick], atol=np.sqrt(k) * 0.05 * 2e-5)
+    dx, dW = dev.put(x), dev.put(W)
+    dy = dev.alloc(rows * out * (2 if out_bf16 else 4))
+    fn = dev.lib.iris_dev_linear_bf16 if out_bf16 else dev.lib.iris_dev_linear_f32
+    dev.lib.iris_dev_linear_backend(1)
+    try:
+        got = run(dev, lambda: fn(dy, dx, dW, rows, k, out), [(dy, (rows, out), np.uint16 if out_bf16 else np.float32)])
+        kernel = dev.dev.last_kernel()
+    finally:
+        dev.lib.iris_dev_linear_backend(0)
+    assert kernel == "linear_mfma"
+    scale = np.sqrt(k) * 0.05
+    if out_bf16:
+        assert np.all(np.abs(O.bf16_to_f32(got) - want) <= np.abs(want) * 2.0 ** -8 * 1.01 + scale * 2e-5)
+    else:
+        assert np.abs(got - want).max() <= scale * 2e-5
+
+
 def test_linear_unaligned_k_uses_the_scalar_kernel(dev, orc):
     rows, k, out = 37, 27, 19                              # k*k*cin of the 3-channel input convolution
     x, W = O.f32_to_bf16(rnd((rows, k), 1)), O.f32_to_bf16(rnd((out, k), 2))

@@ -120,3 +120,29 @@ def test_other_device_operators(orc, gold):
     gamma, beta = (1 + 0.1 * inputs(147, 16)).astype(np.float32), (0.1 * inputs(148, 16)).astype(np.float32)
     np.testing.assert_allclose(orc.dev_group_norm(gimg, gamma, beta, 4, 1e-6, 0), gold["ops_group_norm"], atol=1e-5)
     np.testing.assert_array_equal(orc.dev_upsample2x(inputs(149, 12, 5), 3, 4), gold["ops_upsample2x"])
+
+
+# ---- the metric's own chain at head_dim 128 (configuration C1, full shape), held by the compiled reference
+C1_GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "c1_chain.npz")
+
+
+def test_c1_chain_f32_plumbing(orc):
+    """apply_qk_norm -> apply_rope_2d -> iris_flash_attention of the reference on C1 at full shape (24 x 128, 320
+    tokens; vector written by tests/golden/make_golden.py:c1_chain) against the oracle's f32 chain on the same seeded
+    inputs: <= 1e-4 absolute, the tolerance of the fp32 plumbing configuration."""
+    import workloads as W
+    g = np.load(C1_GOLD, allow_pickle=False)
+    case = W.c1()
+    seq, heads, hd, dim = case["seq"], 24, 128, 3072
+    f = O.bf16_to_f32(case["buf"])
+    q, k, v = (np.ascontiguousarray(f[:, i * dim:(i + 1) * dim]) for i in range(3))
+    qn = orc.head_norm_rope_f32(q.reshape(seq, heads, hd), case["wq"], case["cos"], case["sin"], case["eps"], 0).reshape(seq, dim)
+    kn = orc.head_norm_rope_f32(k.reshape(seq, heads, hd), case["wk"], case["cos"], case["sin"], case["eps"], 0).reshape(seq, dim)
+    rows = g["rows"]
+    assert np.abs(qn[rows] - g["q_rows"]).max() <= 1e-5 and np.abs(kn[rows] - g["k_rows"]).max() <= 1e-5
+    out = orc.attention_flash(qn, kn, v, heads, case["scale"])
+    assert np.abs(out[rows] - g["out_rows"]).max() <= 1e-4
+    np.testing.assert_allclose([out.astype(np.float64).sum(), np.abs(out).astype(np.float64).sum()], g["out_checksum"], rtol=1e-5)
+    # the strided routine the GPU tests compare with, on the same rows
+    strided = orc.attention_strided(qn, kn, v, heads, heads, case["scale"])
+    assert np.abs(strided[rows] - g["out_rows"]).max() <= 1e-4
