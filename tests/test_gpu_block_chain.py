@@ -422,8 +422,11 @@ def test_double_stream_block_full_size(dev, orc):
     assert np.array_equal(snap["h_after"][:, 2 * dim:], snap["h_before"][:, 2 * dim:]), "V columns changed"
     g, w = O.bf16_to_f32(snap["h_after"][:, :2 * dim]), O.bf16_to_f32(want_h[:, :2 * dim])
     ulp = np.maximum(np.abs(w), 2.0 ** -126) * 2.0 ** -7          # one bf16 step at the expected value
-    worst = np.abs(g - w) / ulp
-    assert worst.max() <= 1.0 + 1e-6 or np.abs(g - w).max() <= 1e-5, f"norm+rope off by {worst.max():.3g} bf16 steps"
+    gap = np.abs(g - w)
+    # one rounding of (nearly) the same f32 value: at most one bf16 step apart, except where a*c - b*s cancels to
+    # about zero and the f32 operation order decides the low bits: there the absolute gap is tiny
+    bad = (gap > ulp * 1.01) & (gap > 1e-5)
+    assert not bad.any(), f"norm+rope: {bad.sum()} entries off by more than one bf16 step, worst gap {gap[bad].max():.3g}"
     assert (snap["h_after"][:, :2 * dim] != want_h[:, :2 * dim]).mean() < 0.02, "more than 2 % of the entries differ in the last bit"
     # 3. attention on sampled rows, from the device's normalised rows
     want_att = orc.attention_bf16(snap["h_after"], 3 * dim, 0, dim, 2 * dim, seq, seq, heads, heads, 128, b["scale"], rows=rows)
