@@ -64,18 +64,22 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
     u32x4 raw[kUnroll];
     float4 ct[kUnroll][TN], st[kUnroll][TN];
     uint16_t *ptr[kUnroll];
-    bool isk[kUnroll], later[kUnroll];
+    float4 wv[kUnroll][2];                          /* the norm weights of this lane's 8 dims */
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
         int unit = first + u * (kThreads / 16);
         const bool live = unit < units;
         unit = live ? unit : 0;
-        later[u] = STREAMS && unit >= second.first_unit;
+        const bool later = STREAMS && unit >= second.first_unit;
         /* unit / heads_total; one head per token has no 32-bit magic (it would be 2^32) */
         const int s = heads_total == 1 ? unit : (int)__umulhi((uint32_t)unit, magic);
         const int h = unit - s * heads_total;
-        isk[u] = h >= q_heads;
-        uint16_t *base = isk[u] ? xk + (size_t)(h - q_heads) * 128 : xq + (size_t)h * 128;
+        const bool isk = h >= q_heads;
+        uint16_t *base = isk ? xk + (size_t)(h - q_heads) * 128 : xq + (size_t)h * 128;
+        /* the vector's weights: Q's or K's, of the first or (STREAMS) of the second row range */
+        const float *wsel = isk ? (later ? second.wk : wk) : (later ? second.wq : wq);
+        wv[u][0] = *reinterpret_cast<const float4 *>(wsel + sub * 8);
+        wv[u][1] = *reinterpret_cast<const float4 *>(wsel + sub * 8 + 4);
         ptr[u] = live ? base + (size_t)s * ld + sub * 8 : nullptr;
         raw[u] = live ? *reinterpret_cast<const u32x4 *>(ptr[u]) : u32x4{0, 0, 0, 0};
         const float *cp = rope_cos + (size_t)s * 64 + tcol;
@@ -86,28 +90,6 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
             st[u][i] = *reinterpret_cast<const float4 *>(sp + 4 * i);
         }
     }
-    /* the norm weights of this lane's 8 dims (Q and, when present, K) */
-    float wq8[8], wk8[8];
-    {
-        const float4 a0 = *reinterpret_cast<const float4 *>(wq + sub * 8);
-        const float4 a1 = *reinterpret_cast<const float4 *>(wq + sub * 8 + 4);
-        const float *wks = heads_total > q_heads ? wk : wq;
-        const float4 b0 = *reinterpret_cast<const float4 *>(wks + sub * 8);
-        const float4 b1 = *reinterpret_cast<const float4 *>(wks + sub * 8 + 4);
-        wq8[0] = a0.x; wq8[1] = a0.y; wq8[2] = a0.z; wq8[3] = a0.w; wq8[4] = a1.x; wq8[5] = a1.y; wq8[6] = a1.z; wq8[7] = a1.w;
-        wk8[0] = b0.x; wk8[1] = b0.y; wk8[2] = b0.z; wk8[3] = b0.w; wk8[4] = b1.x; wk8[5] = b1.y; wk8[6] = b1.z; wk8[7] = b1.w;
-    }
-    float wq8b[8], wk8b[8];                         /* the second stream's pair */
-    if (STREAMS) {
-        const float4 a0 = *reinterpret_cast<const float4 *>(second.wq + sub * 8);
-        const float4 a1 = *reinterpret_cast<const float4 *>(second.wq + sub * 8 + 4);
-        const float *wks = heads_total > q_heads ? second.wk : second.wq;
-        const float4 b0 = *reinterpret_cast<const float4 *>(wks + sub * 8);
-        const float4 b1 = *reinterpret_cast<const float4 *>(wks + sub * 8 + 4);
-        wq8b[0] = a0.x; wq8b[1] = a0.y; wq8b[2] = a0.z; wq8b[3] = a0.w; wq8b[4] = a1.x; wq8b[5] = a1.y; wq8b[6] = a1.z; wq8b[7] = a1.w;
-        wk8b[0] = b0.x; wk8b[1] = b0.y; wk8b[2] = b0.z; wk8b[3] = b0.w; wk8b[4] = b1.x; wk8b[5] = b1.y; wk8b[6] = b1.z; wk8b[7] = b1.w;
-    }
-
     /* Phase 2: normalise, rotate, store. */
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
@@ -117,12 +99,7 @@ k_norm_rope_hd128(uint16_t *__restrict__ xq, uint16_t *__restrict__ xk, int ld,
         cv[4] = ct[u][TN - 1].x; cv[5] = ct[u][TN - 1].y; cv[6] = ct[u][TN - 1].z; cv[7] = ct[u][TN - 1].w;
         sv[0] = st[u][0].x; sv[1] = st[u][0].y; sv[2] = st[u][0].z; sv[3] = st[u][0].w;
         sv[4] = st[u][TN - 1].x; sv[5] = st[u][TN - 1].y; sv[6] = st[u][TN - 1].z; sv[7] = st[u][TN - 1].w;
-        float w8[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            w8[i] = isk[u] ? wk8[i] : wq8[i];
-            if (STREAMS) w8[i] = later[u] ? (isk[u] ? wk8b[i] : wq8b[i]) : w8[i];
-        }
+        const float w8[8] = {wv[u][0].x, wv[u][0].y, wv[u][0].z, wv[u][0].w, wv[u][1].x, wv[u][1].y, wv[u][1].z, wv[u][1].w};
         const u32x4 out = nr_vector_hd128<SPLIT>(raw[u], w8, cv, sv, eps, sub);
         /* Write-through store (sc0 sc1): the rows leave the L2 as they are produced instead of at the
          * end-of-kernel write-back, 2-5 % faster on 59-118 MB calls whether the rows were cached or not.
