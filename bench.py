@@ -402,7 +402,7 @@ def other_ops(dev, hip, stream, rng, settle_ms=0.0):
     y = lib.iris_dev_alloc(rows * 27648 * 4)
     for k, n in ((3072, 9216), (3072, 3072), (3072, 18432), (9216, 3072), (3072, 27648), (12288, 3072)):
         for name, fn in (("linear_f32", lib.iris_dev_linear_f32), ("linear_bf16", lib.iris_dev_linear_bf16)):
-            for backend in (0, 1):            # 0: vendor GEMM library when present (the default), 1: own MFMA kernel
+            for backend in (2, 0):            # 2: the vendor GEMM library when present (the yardstick), 0: own MFMA kernel (the default)
                 lib.iris_dev_linear_backend(backend)
                 ms = timed(lambda i: fn(y, x, W, rows, k, n), 5)
                 res.append({"op": name, "kernel": dev.last_kernel(), "shape": f"{rows}x{k}->{n}", "us": round(ms * 1e3, 1),
@@ -421,7 +421,7 @@ def other_ops(dev, hip, stream, rng, settle_ms=0.0):
 
         def one_call(i):
             lib.iris_dev_linear_bf16_qknorm(y, x, W, rows, dim, n, heads, heads, 128, w1, w1, cos, sin, 1e-6, 0)
-        for backend in (0, 1):
+        for backend in (2, 0):
             lib.iris_dev_linear_backend(backend)
             for name, fn in (("linear_bf16 + 2 x head_norm_rope", three_calls), ("linear_bf16_qknorm", one_call)):
                 ms = timed(fn, 5)

@@ -194,8 +194,8 @@ void iris_dev_attention_qnorm(uint16_t *out, int ldo,
  * (iris_transformer_flux.c:3795-3800 and 3833-3837, iris_transformer_flux3.c:692-694,
  * iris_transformer_zimage.c:1947-1949, iris_qwen3.c:1589-1593), which all issue exactly these three calls. The
  * library's own GEMM can normalise each 256 x 256 output tile while it still sits in the LDS, which saves the
- * pass that reads and rewrites the Q and K rows: that one-launch kernel runs when the own GEMM is selected
- * (iris_dev_linear_backend(1)) or the vendor library is absent, for head_dim 128, rows >= 256, out >= 256 and
+ * pass that reads and rewrites the Q and K rows: that one-launch kernel runs unless the vendor GEMM is selected
+ * (iris_dev_linear_backend(2)) and present, for head_dim 128, rows >= 256, out >= 256 and
  * a multiple of 128, in a multiple of 64 and 16-byte aligned operands; its bits are those of the two calls
  * above on the own GEMM. Otherwise the entry issues the two calls itself (the vendor GEMM followed by the norm
  * kernel is the faster pair where that library is present). */
@@ -216,10 +216,10 @@ int iris_dev_last_error(void);
  * call used: a static string such as "fa_hd128" or "generic". */
 const char *iris_dev_last_kernel(void);
 
-/* Which GEMM runs the linear layers. 0 (default): the vendor library hipBLASLt when it can be
- * opened at run time and takes the problem, this library's own MFMA kernel otherwise
- * (the reference's backend calls cuBLAS / hipBLAS for them, iris_cuda.cu:456-505);
- * 1: always the own kernel. No counterpart in the reference. */
+/* Which GEMM runs the linear layers. 0 (default) and 1: this library's own MFMA kernels. 2: the vendor
+ * library hipBLASLt where it can be opened at run time and takes the problem (the reference's backend calls
+ * cuBLAS / hipBLAS for them, iris_cuda.cu:456-505), the own kernels otherwise: the yardstick the benchmark
+ * measures the own kernels against, not a production path. No counterpart in the reference. */
 void iris_dev_linear_backend(int which);
 
 #ifdef __cplusplus

@@ -417,15 +417,15 @@ void iris_dev_f32_to_bf16(uint16_t *dst, const float *src, size_t n) {
     LAUNCH("f32_to_bf16", iris_hip_f32_to_bf16(g_stream, dst, src, n));
 }
 
-/* Plain GEMMs go to the vendor library when it is there and takes the problem (aligned operands,
- * in % 8 == 0), to this library's own MFMA kernel otherwise. iris_dev_linear_backend(1) pins the
- * own kernel. */
+/* Plain GEMMs run on this library's own MFMA kernels. iris_dev_linear_backend(2) sends them to the vendor
+ * library instead, where it can be opened and takes the problem (aligned operands, in % 8 == 0): the yardstick
+ * the benchmark compares the own kernels with. 0 and 1 select the own kernels. */
 static int g_linear_backend = 0;
 
-void iris_dev_linear_backend(int which) { g_linear_backend = which == 1 ? 1 : 0; }
+void iris_dev_linear_backend(int which) { g_linear_backend = which == 2 ? 2 : 0; }
 
 static int linear_by_library(void *y, int out_bf16, const uint16_t *x, const uint16_t *W, int rows, int in, int out) {
-    if (g_linear_backend != 0 || in % 8 != 0 || !aligned(y, 16) || !aligned(x, 16) || !aligned(W, 16)) return 0;
+    if (g_linear_backend != 2 || in % 8 != 0 || !aligned(y, 16) || !aligned(x, 16) || !aligned(W, 16)) return 0;
     if (iris_lt_linear(g_stream, y, out_bf16, x, W, rows, in, out) != 0) return 0;
     g_last_kernel = "linear_hipblaslt";
     return 1;
@@ -459,11 +459,9 @@ void iris_dev_linear_bf16_qknorm(uint16_t *y, const uint16_t *x, const uint16_t 
         return;
     }
     if (!need_ready("linear_qknorm")) return;
-    /* With the vendor GEMM selected and present, its linear layer followed by the norm kernel is the faster pair
-     * (4608 rows, 3072 -> 9216: 215 us against 225 us for the one-launch kernel, whose GEMM is the library's
-     * own: 199 + 17 against 220 + 7); with the own GEMM selected the one launch saves 11 us of 238. */
+    /* With the vendor GEMM selected and present, the entry is its linear layer followed by the norm kernel. */
     int one_launch = head_dim == 128 && q_heads + k_heads > 0 &&
-                     (g_linear_backend != 0 || !iris_lt_available() || in % 8 != 0);
+                     (g_linear_backend != 2 || !iris_lt_available() || in % 8 != 0);
     if (one_launch) {
         int err = iris_hip_linear_bf16_qknorm(g_stream, y, x, W, rows, in, out, q_heads * 128, k_heads * 128, wq, wk,
                                               rope_cos, rope_sin, eps, split_half != 0);

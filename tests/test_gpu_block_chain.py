@@ -87,9 +87,9 @@ def device_block(dev, b, q_norm_inside_attention, norm_inside_projection=False):
     return got, kernel
 
 
-@pytest.mark.parametrize("seq,heads,mlp,backend", [(80, 4, 1024, 0), (333, 3, 768, 1), (600, 2, 512, 1)])
+@pytest.mark.parametrize("seq,heads,mlp,backend", [(80, 4, 1024, 2), (333, 3, 768, 0), (600, 2, 512, 0)])
 def test_single_stream_block_chain(dev, orc, seq, heads, mlp, backend):
-    """backend 0: linear layers on the vendor GEMM when present; 1: on the library's own kernels (333 and 600 rows
+    """backend 2: linear layers on the vendor GEMM when present; 0: on the library's own kernels, the default (333 and 600 rows
     reach the 256 x 256 kernel with ragged edges)."""
     b = make_block(seq + heads, seq, heads, mlp)
     dev.lib.iris_dev_linear_backend(backend)
@@ -106,10 +106,10 @@ def test_single_stream_block_chain(dev, orc, seq, heads, mlp, backend):
     assert mx <= 3e-2 and mean <= 3e-3, f"max-abs {mx:.4g}, mean-abs {mean:.4g}"
     assert np.array_equal(got, fused), "the block with Q normalised inside attention differs from the three-call block"
     # the projection that normalises its own Q and K columns (rows >= 256: one launch; fewer: the two steps)
-    assert projection == ("linear_mfma_qknorm" if seq >= 256 and backend == 1 else "norm_rope_hd128")
+    assert projection == ("linear_mfma_qknorm" if seq >= 256 and backend == 0 else "norm_rope_hd128")
     mx, mean = error_stats(one_launch - b["x"], want - b["x"])
     assert mx <= 3e-2 and mean <= 3e-3, f"projection with norm: max-abs {mx:.4g}, mean-abs {mean:.4g}"
-    if backend == 1 or projection == "norm_rope_hd128":
+    if backend == 0 or projection == "norm_rope_hd128":
         assert np.array_equal(got, one_launch), "the block with the norm inside the projection differs from the three-call block"
 
 
@@ -358,7 +358,7 @@ def oracle_double_block(orc, b):
     return x, x_mid
 
 
-@pytest.mark.parametrize("txt,img,heads,mlp,backend", [(48, 272, 3, 768, 1), (37, 219, 2, 512, 0), (300, 724, 2, 0, 1)])
+@pytest.mark.parametrize("txt,img,heads,mlp,backend", [(48, 272, 3, 768, 0), (37, 219, 2, 512, 2), (300, 724, 2, 0, 0)])
 def test_double_stream_block_chain(dev, orc, txt, img, heads, mlp, backend):
     """The double-stream block as the reference issues it: FOUR norm+rope launches on row sub-ranges of the joint
     q | k | v rows (text rows, image rows; Q and K each) with the stream's own weight pair and the tables offset to the
@@ -397,7 +397,7 @@ def test_double_stream_block_full_size(dev, orc):
     the stream boundary among them."""
     b = make_double_block(7, 512, 4096, 24, 0)
     seq, dim, heads, txt = b["seq"], b["dim"], b["heads"], b["txt"]
-    dev.lib.iris_dev_linear_backend(1)
+    dev.lib.iris_dev_linear_backend(0)
     try:
         got, kernels, snap = device_double_block(dev, b, snapshots=True)
     finally:
@@ -442,7 +442,7 @@ def test_double_stream_block_full_size(dev, orc):
         assert mx <= 3e-2 and mean <= 3e-3, f"residual update, stream {m}: max-abs {mx:.4g}, mean-abs {mean:.4g}"
     assert np.array_equal(got, snap["x_mid"])
     # the one-launch form of the four norm calls: same rows, bit for bit
-    dev.lib.iris_dev_linear_backend(1)
+    dev.lib.iris_dev_linear_backend(0)
     try:
         _, _, snap_one = device_double_block(dev, b, fused_qk="streams", snapshots=True)
     finally:

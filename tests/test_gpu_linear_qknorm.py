@@ -99,14 +99,14 @@ def test_one_launch_matches_oracle_chain_and_own_two_calls(dev, orc, rows, k, q_
     assert not np.array_equal(got[:, :qk], plain[:, :qk])
 
 
-def test_default_backend_against_oracle(dev, orc):
-    """With the vendor GEMM selected and present the entry issues that GEMM and the norm kernel; without it the
+def test_vendor_backend_against_oracle(dev, orc):
+    """With the vendor GEMM selected (2) and present the entry issues that GEMM and the norm kernel; without it the
     one-launch kernel. Either way the oracle's chain is the yardstick."""
     c = make(5, 512, 256, 4, 4, 512)
-    got, kernel = run(dev, c, True, 0, 0)
+    got, kernel = run(dev, c, True, 0, 2)
     assert kernel in ("norm_rope_hd128", "linear_mfma_qknorm")
-    assert_parity(bf16_to_f32(got), bf16_to_f32(oracle_chain(orc, c, 0)), "default backend")
-    two, _ = run(dev, c, False, 0, 0)
+    assert_parity(bf16_to_f32(got), bf16_to_f32(oracle_chain(orc, c, 0)), "vendor backend")
+    two, _ = run(dev, c, False, 0, 2)
     assert np.array_equal(got, two)
 
 
@@ -123,7 +123,7 @@ TWO_STEP = [
 @pytest.mark.parametrize("rows,k,q_heads,k_heads,extra,hd,split", TWO_STEP)
 def test_other_shapes_run_the_two_steps(dev, orc, rows, k, q_heads, k_heads, extra, hd, split):
     c = make(rows + hd, rows, k, q_heads, k_heads, extra, hd)
-    for backend in (0, 1):
+    for backend in (2, 0):
         got, kernel = run(dev, c, True, split, backend)
         assert kernel.startswith("norm_rope")
         two, _ = run(dev, c, False, split, backend)
