@@ -85,7 +85,7 @@ def traffic_on_file():
             if line.startswith("total_bytes_per_launch:"):
                 nbytes = int(line.split(":")[1].strip().replace(",", ""))
             if line.startswith("kernel_source_sha256:"):
-                sha = line.split(":")[1].strip()
+                sha = line.split(":")[1].split()[0]
     except OSError:
         return None, None, None
     return nbytes, TRAFFIC_PROFILE, sha != source_sha256()
@@ -876,7 +876,7 @@ def main():
                      "launch_ms_median": round(float(np.median(att)), 4), "launch_ms_min": round(float(np.min(att)), 4),
                      "single_launch_ms": round(att_single, 4),
                      "flops_per_launch": flops},
-        "norm_rope": {"kernel": "k_norm_rope_hd128", "bound": "hbm", "unit": "GB/s", "peak": PEAK_HBM_GBPS,
+        "norm_rope": {"kernel": "k_norm_rope_hd128<false, false, false>", "bound": "hbm", "unit": "GB/s", "peak": PEAK_HBM_GBPS,
                       "bytes_per_call": q_bytes,
                       "q_call_us": round(nr_q_ms * 1e3, 2), "q_call_gbps": round(q_bytes / (nr_q_ms * 1e-3) / 1e9, 1),
                       "q_call_frac": round(q_bytes / (nr_q_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),

@@ -83,3 +83,23 @@ def test_linear_layers_of_the_models_take_the_four_wave_kernel_in_the_width_that
     assert linear_plan(700, 256, 1000) == (3, 256) or linear_plan(700, 256, 1000)[0] == 3
     assert linear_plan(64, 128, 64)[0] == 1 and linear_plan(37, 27, 19)[0] == 0
     assert linear_plan(512, 256, 258, 4)[0] == 2             # f32 rows of 258 columns cannot take 16-byte stores
+
+
+def test_profile_summaries_say_which_source_they_were_taken_on():
+    """Every summary under profiles/ names the commit and the hash of the kernel source it was measured on, and
+    bench.py can tell from the C2 counter file whether its traffic figure belongs to the kernel source in the tree."""
+    import glob
+    import os
+    import re
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    files = sorted(glob.glob(os.path.join(root, "profiles", "*.txt")))
+    assert len(files) >= 10
+    for path in files:
+        text = open(path).read()
+        assert re.search(r"^taken_on_commit: [0-9a-f]{40}$", text, re.M), path
+        assert re.search(r"^kernel_source_sha256: [0-9a-f]{16}\s+\(iris_c_amd/csrc/\w+\.hip\)$", text, re.M), path
+    sys.path.insert(0, root)
+    import bench
+    nbytes, source, stale = bench.traffic_on_file()
+    assert nbytes and nbytes > 113_246_208 and source.endswith("hbm_traffic.txt") and stale in (True, False)
