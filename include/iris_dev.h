@@ -64,8 +64,7 @@ void iris_dev_head_norm_rope(uint16_t *x, int ld, const float *w,
  * 0 = ignored key, or NULL. A query with no valid key gives a zero row
  * (reference iris_cuda.cu:531, 650, 676).
  * Every combination of heads / kv_heads / head_dim / stride / alignment is answered, as in the
- * reference, with one limit: head_dim <= 2048 (larger is reported as an error; the reference's
- * GEMM-based fallback has no such limit, none of its models comes near it). head_dim 128, 256
+ * reference (its fallback is two GEMMs, iris_cuda.cu:897-936, with no limit on head_dim). head_dim 128, 256
  * and 512 on 16-byte aligned rows run on the matrix cores directly, any other head_dim <= 512 or
  * alignment through a padded, aligned private copy of q, k, v; the rest (head_dim > 512,
  * scale <= 0, more than 250000 masked keys) on a scalar kernel.

@@ -48,14 +48,17 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 /* head_dim beyond MAX_HD: the dot products are accumulated over chunks of MAX_HD dims (the K tile in LDS
  * holds one chunk at a time), and the output is produced MAX_HD dims at a time, each such pass walking the
- * keys again with its own softmax state. */
+ * keys again with its own softmax state.
+ * Q_IN_LDS: the workgroup's 8 queries are kept in the LDS as f32 (head_dim <= 2048: 64 KB); beyond that they are
+ * read from global memory where they are used (they stay in the caches: every lane reads the same addresses). */
+template <bool Q_IN_LDS>
 __global__ void __launch_bounds__(64)
 k_attention_generic(uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k, const uint16_t *v,
                     int ldq, int ldi, int seq_q, int seq_k, int kv_group, int hd, int kstride, float scale,
                     int causal, const int *key_mask) {
     extern __shared__ __align__(16) unsigned char smem[];
-    float *qs = reinterpret_cast<float *>(smem);                 /* [QB][hd] */
-    float *ps = qs + QB * hd;                                     /* [QB][KT] */
+    float *qs = reinterpret_cast<float *>(smem);                 /* [QB][hd], or nothing */
+    float *ps = qs + (Q_IN_LDS ? QB * hd : 0);                    /* [QB][KT] */
     uint16_t *kt = reinterpret_cast<uint16_t *>(ps + QB * KT);    /* [KT][kstride]: one chunk of dims */
 
     const int lane = threadIdx.x;
@@ -63,9 +66,11 @@ k_attention_generic(uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k
     const int q0 = blockIdx.x * QB;
     const int nq = min(QB, seq_q - q0);
 
-    for (int idx = lane; idx < QB * hd; idx += 64) {
-        int qq = idx / hd, d = idx - qq * hd;
-        qs[idx] = qq < nq ? bf2f(q[(size_t)(q0 + qq) * ldq + (size_t)head * hd + d]) : 0.0f;
+    if (Q_IN_LDS) {
+        for (int idx = lane; idx < QB * hd; idx += 64) {
+            int qq = idx / hd, d = idx - qq * hd;
+            qs[idx] = qq < nq ? bf2f(q[(size_t)(q0 + qq) * ldq + (size_t)head * hd + d]) : 0.0f;
+        }
     }
 
     int k_end = seq_k;
@@ -98,9 +103,15 @@ k_attention_generic(uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k
                 const uint16_t *kv = kt + lane * kstride;
 #pragma unroll
                 for (int qq = 0; qq < QB; qq++) {
-                    const float *qv = qs + qq * hd + dc;
                     float part = dot[qq];
-                    for (int d = 0; d < cw; d++) part = fmaf(qv[d], bf2f(kv[d]), part);
+                    if (Q_IN_LDS) {
+                        const float *qv = qs + qq * hd + dc;
+                        for (int d = 0; d < cw; d++) part = fmaf(qv[d], bf2f(kv[d]), part);
+                    } else {
+                        /* rows past the last query repeat it: their scores are never used */
+                        const uint16_t *qg = q + (size_t)(q0 + min(qq, nq - 1)) * ldq + (size_t)head * hd + dc;
+                        for (int d = 0; d < cw; d++) part = fmaf(bf2f(qg[d]), bf2f(kv[d]), part);
+                    }
                     dot[qq] = part;
                 }
             }
@@ -210,18 +221,26 @@ extern "C" int iris_hip_attention_generic(void *stream, uint16_t *out, int ldo, 
     const int chunk = head_dim < MAX_HD ? head_dim : MAX_HD;
     int kstride = ((chunk + 1) & ~1) + 2;
     if ((kstride / 2) % 2 == 0) kstride += 2;
-    const size_t smem = (size_t)QB * head_dim * 4 + (size_t)QB * KT * 4 + (size_t)KT * kstride * 2;
-    if (smem > 160 * 1024) return (int)hipErrorInvalidValue;      /* the caller keeps head_dim <= IRIS_ATTENTION_MAX_HEAD_DIM */
+    const bool q_in_lds = head_dim <= IRIS_ATTENTION_Q_IN_LDS_MAX_HEAD_DIM;
+    const size_t smem = (q_in_lds ? (size_t)QB * head_dim * 4 : 0) + (size_t)QB * KT * 4 + (size_t)KT * kstride * 2;
+    if (smem > 160 * 1024) return (int)hipErrorInvalidValue;
     static bool big_lds = false;
     if (!big_lds) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_attention_generic),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_attention_generic<true>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_attention_generic<false>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return (int)e;
         big_lds = true;
     }
     dim3 grid((seq_q + QB - 1) / QB, heads);
-    hipLaunchKernelGGL(k_attention_generic, grid, dim3(64), smem, (hipStream_t)stream, out, ldo, q, k, v,
-                       ldq, ldi, seq_q, seq_k, heads / kv_heads, head_dim, kstride, scale, causal, key_mask);
+    if (q_in_lds)
+        hipLaunchKernelGGL(k_attention_generic<true>, grid, dim3(64), smem, (hipStream_t)stream, out, ldo, q, k, v,
+                           ldq, ldi, seq_q, seq_k, heads / kv_heads, head_dim, kstride, scale, causal, key_mask);
+    else
+        hipLaunchKernelGGL(k_attention_generic<false>, grid, dim3(64), smem, (hipStream_t)stream, out, ldo, q, k, v,
+                           ldq, ldi, seq_q, seq_k, heads / kv_heads, head_dim, kstride, scale, causal, key_mask);
     return (int)hipGetLastError();
 }
 

@@ -70,9 +70,10 @@ int iris_hip_fa_sliced(void *stream, uint16_t *out, int ldo, const uint16_t *q,
                        int heads, int kv_heads, int head_dim, float scale, int causal,
                        const int *key_mask);
 
-/* Any head_dim <= IRIS_ATTENTION_MAX_HEAD_DIM (the 8 queries of a workgroup are kept in LDS as f32),
- * any stride / alignment / scale; the rows of q may have a stride (ldq) of their own. Correctness path. */
-#define IRIS_ATTENTION_MAX_HEAD_DIM 2048
+/* Any head_dim (up to IRIS_ATTENTION_Q_IN_LDS_MAX_HEAD_DIM the 8 queries of a workgroup are kept in LDS as f32,
+ * beyond it they are read from global memory), any stride / alignment / scale; the rows of q may have a stride
+ * (ldq) of their own. Correctness path. */
+#define IRIS_ATTENTION_Q_IN_LDS_MAX_HEAD_DIM 2048
 int iris_hip_attention_generic(void *stream, uint16_t *out, int ldo, const uint16_t *q, int ldq,
                                const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
                                int seq_k, int heads, int kv_heads, int head_dim, float scale,

@@ -485,10 +485,12 @@ def test_padded_copy_with_fewer_queries_than_keys_and_large_sizes(dev, orc):
         assert_close(O.bf16_to_f32(out[:seq_q])[rows], want, f"padded copy {seq_q}x{seq_k}")
 
 
-@pytest.mark.parametrize("hd,heads,kv,causal", [(640, 2, 1, True), (1024, 1, 1, False), (2048, 1, 1, False), (1100, 2, 2, False)])
+@pytest.mark.parametrize("hd,heads,kv,causal", [(640, 2, 1, True), (1024, 1, 1, False), (2048, 1, 1, False), (1100, 2, 2, False),
+                                                (2050, 1, 1, True), (2304, 2, 1, False), (5000, 1, 1, False)])
 def test_head_dims_beyond_512_on_the_scalar_kernel(dev, orc, hd, heads, kv, causal):
-    """The reference answers any head_dim (its fallback is two GEMMs); here sizes beyond the matrix-core kernels'
-    512 go to the scalar kernel, which walks the dims in chunks of 512, up to 2048."""
+    """The reference answers any head_dim (its fallback is two GEMMs, iris_cuda.cu:897-936); here sizes beyond the
+    matrix-core kernels' 512 go to the scalar kernel, which walks the dims in chunks of 512: up to 2048 with the
+    workgroup's queries in the LDS, beyond that reading them from global memory. No limit on head_dim."""
     seq = 70
     buf, ldi = random_case(hd, seq, seq, heads, kv, hd=hd)
     qd, kd = heads * hd, kv * hd
@@ -516,6 +518,6 @@ def test_bad_arguments_are_reported_not_fatal(dev):
     dev.lib.iris_dev_last_error()
     dev.lib.iris_dev_attention(d, 384, d, d, d, ldi, 8, 8, 3, 2, 128, 0.1, 0, None)    # 3 % 2 != 0
     assert dev.lib.iris_dev_last_error() != 0
-    dev.lib.iris_dev_attention(d, 4096, d, d, d, ldi, 8, 8, 1, 1, 2049, 0.1, 0, None)   # head_dim beyond the limit
+    dev.lib.iris_dev_attention(d, 4096, d, d, d, ldi, 8, 8, 1, 1, 0, 0.1, 0, None)      # head_dim must be positive
     assert dev.lib.iris_dev_last_error() != 0
     dev.free_all()
