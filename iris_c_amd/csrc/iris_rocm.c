@@ -231,8 +231,8 @@ static void norm_rope_streams(uint16_t *xq, uint16_t *xk, int ld, const float *w
                               int k_heads, int head_dim, float eps, int split_half) {
     if (!need_ready("head_norm_rope")) return;
     if (seq <= 0 || q_heads + k_heads <= 0) return;
-    if (head_dim <= 0 || (head_dim & 1) || head_dim > 1024) {
-        fail(-1, "head_norm_rope", "head_dim must be even and <= 1024");
+    if (head_dim <= 0 || (head_dim & 1)) {                   /* the reference takes powers of two up to 2048 (iris_cuda.cu:445-453) */
+        fail(-1, "head_norm_rope", "head_dim must be even");
         return;
     }
     int fast = head_dim == 128 && ld % 8 == 0 && aligned(xq, 16) && aligned(wq, 16) &&

@@ -112,7 +112,7 @@ def test_empty_input_is_a_no_op(dev):
     assert np.array_equal(dev.norm_rope(buf, 256, 0, w, t, t, 0, 2, 128, 1e-6, 0), buf)
 
 
-@pytest.mark.parametrize("hd,split", [(64, 0), (64, 1), (256, 0), (96, 1)])
+@pytest.mark.parametrize("hd,split", [(64, 0), (64, 1), (256, 0), (96, 1), (2048, 0), (2050, 1)])
 def test_other_head_dims_take_the_generic_kernel(dev, orc, hd, split):
     rng = np.random.default_rng(hd)
     seq, heads = 9, 3
