@@ -112,3 +112,41 @@ def test_a_layout_that_needs_scratch_is_refused_during_capture_until_the_scratch
         assert np.array_equal(dev.get(out, (seq, heads * hd), np.uint16), want)
     g.rt.hipGraphExecDestroy(run)
     dev.free_all()
+
+
+def test_double_stream_step_replayed_from_a_graph():
+    """The joint block's step with the one-launch norm of both streams (iris_dev_head_norm_rope_qk_streams: text rows
+    and image rows with their own weight pairs) and attention, captured once and replayed: every replay equals the
+    eager step bit for bit."""
+    case = W.c2(shrink=4)
+    dev, g = Dev(), Graphs()
+    lib, stream = dev.lib, _vp(dev.lib.iris_dev_stream())
+    seq, ldi, qd, kd = case["seq"], case["ldi"], case["q_dim"], case["kv_dim"]
+    txt = 512 // 4
+    rows, out = dev.put(case["buf"]), dev.alloc(seq * case["ldo"] * 2)
+    wq, wk, cos, sin = dev.put(case["wq"]), dev.put(case["wk"]), dev.put(case["cos"]), dev.put(case["sin"])
+    wq2, wk2 = dev.put(case["wq"][::-1].copy()), dev.put(case["wk"][::-1].copy())
+
+    def step():
+        lib.iris_dev_head_norm_rope_qk_streams(rows, ptr_add(rows, 2 * qd), ldi, wq, wk, wq2, wk2, txt, cos, sin, seq, case["heads"],
+                                               case["kv_heads"], 128, case["eps"], 0)
+        lib.iris_dev_attention(out, case["ldo"], rows, ptr_add(rows, 2 * qd), ptr_add(rows, 2 * (qd + kd)), ldi, seq, seq,
+                               case["heads"], case["kv_heads"], 128, case["scale"], 0, None)
+
+    step()
+    dev.check()
+    want = dev.get(out, (seq, case["ldo"]), np.uint16)
+    assert want.any()
+    run = g.capture(stream, step)
+    dev.check()
+    host = np.ascontiguousarray(case["buf"])
+    for replay in range(3):
+        lib.iris_dev_upload(rows, host.ctypes.data_as(_vp), host.nbytes)
+        junk = np.full((seq, case["ldo"]), 0x7fc0 + replay, np.uint16)
+        lib.iris_dev_upload(out, junk.ctypes.data_as(_vp), junk.nbytes)
+        assert g.rt.hipGraphLaunch(run, stream) == 0
+        lib.iris_dev_sync()
+        dev.check()
+        assert np.array_equal(dev.get(out, (seq, case["ldo"]), np.uint16), want), f"replay {replay} differs from the eager step"
+    g.rt.hipGraphExecDestroy(run)
+    dev.free_all()
