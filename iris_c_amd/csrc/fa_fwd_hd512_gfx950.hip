@@ -1,0 +1,500 @@
+/*
+ * Flash-attention forward for gfx950, head_dim 512, no mask, not causal: the
+ * VAE mid-block attention of the reference (one head of 512 over every latent
+ * position, iris_vae.c:1112-1124; operator contract iris_dev.h:83-92). bf16
+ * in, f32 accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16).
+ *
+ * One wave per SIMD, each with the whole register file: a wave owns 32 queries
+ * and all 512 output dims of them, O^T as 64 accumulator blocks of 16 dims x 16
+ * queries = 256 registers that live in AGPRs (the products that update them are
+ * asm statements, so that they stay there), Q^T as 32 B operands = 128 VGPRs.
+ * No wave ever needs another wave's partial scores: the only thing the four
+ * waves of a workgroup (128 queries) share is the K and V tiles in the LDS.
+ * Both products are transposed as in the head_dim-128 kernel, S^T = K Q^T and
+ * O^T += V^T P^T, so a query is a column of every accumulator, its running
+ * max, bound and rescale factor are per-lane scalars, and exp2(S^T) rounded to
+ * bf16 is the B operand of the second product without leaving the registers.
+ * The row sum comes from one more product per tile with an all-ones A operand.
+ *
+ * Tiles of 32 keys: K and V tile are 32 KB each, two stages of each = 128 KB of
+ * LDS, filled by global_load_lds_dwordx4 (a wave has no registers to stage
+ * them through): one instruction moves one 1 KB tile row, each wave 8 rows of
+ * K and 8 of V per tile, spread over the k-steps of the score product. The
+ * loop is skewed by one tile: turn t multiplies the scores of tile t + 1 and
+ * the values of tile t, so that K of tile t + 2 and V of tile t + 1 (requested
+ * at the start of the turn into the stages the previous turn read last) have a
+ * whole turn to arrive; one barrier per turn. Rows are unpadded; the 16 B
+ * chunk c of row r sits in slot c ^ 2 (r % 8) of its 256 B group, the
+ * permutation applied to the source address of the lane that fills the slot
+ * (same conflict-free pattern as the head_dim-128 kernel: a row is a multiple
+ * of 256 B there and here).
+ *
+ * 128 queries per workgroup make few workgroups (16384 tokens: 128 for 256
+ * CUs), so the keys of a head may be cut into `splits` ranges, one workgroup
+ * per (query tile, range); these write their unnormalised O (f32), running max
+ * and row sum to a scratch buffer and k_fa_hd512_merge combines them.
+ */
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "iris_kernels_hip.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int HD = 512;
+constexpr int BN = 32;              /* keys per tile */
+constexpr int BM = 128;             /* queries per workgroup */
+constexpr int THREADS = 256;
+constexpr int TILE = BN * HD;       /* elements of a K (or V) tile: 32 KB */
+constexpr int XCDS = 8;
+constexpr size_t LDS_BYTES = 4 * (size_t)TILE * sizeof(uint16_t);
+constexpr float RESCALE_THRESHOLD = 8.0f;   /* log2 units */
+
+/* Every lambda below is inlined by the always-inline pass, before anything else runs: a closure that is only
+ * inlined later keeps what it captured (the accumulators) in memory. */
+#define INLINE __attribute__((always_inline))
+
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    f32x2 p = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2));
+}
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    return __builtin_elementwise_maximum(__builtin_elementwise_maximum(a, b), c);
+}
+/* max over the four lanes l%16, +16, +32, +48, which share a query */
+__device__ __forceinline__ float quad_group_max(float v) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    const float t = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ int swz(int row) { return 2 * (row & 7); }
+__device__ __forceinline__ uint32_t lds_address(const uint16_t *p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+__device__ __forceinline__ const uint16_t *scalar_ptr(const uint16_t *p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const uint16_t *)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
+/* Where the partial results of a key range live: [range][head][query] rows of 512 f32, and (max, sum) pairs. */
+struct Partials {
+    float *o, *ml;
+};
+
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+
+template <bool SPLIT>
+__global__ void __launch_bounds__(THREADS, 1)
+k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ q,
+               const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
+               int seq_q, int seq_k, int heads, int q_tiles, int splits, int tiles_per_split,
+               int total_work, int work_per_xcd, int kv_group, float scale_log2, Partials part) {
+    extern __shared__ __align__(16) uint16_t lds[];     /* K stage 0, 1 | V stage 0, 1 */
+
+    const int work = (blockIdx.x % XCDS) * work_per_xcd + blockIdx.x / XCDS;
+    if (work >= total_work) return;
+    const int qt = work % q_tiles, rest = work / q_tiles;
+    const int split = rest % splits, head = rest / splits;
+    const int kvh = head / kv_group;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;       /* 16x16 block: column li, row group lg */
+    const int wq0 = qt * BM + 32 * wave, qrow0 = wq0 + li;
+
+    const uint16_t *kbase = scalar_ptr(k + (size_t)kvh * HD);
+    const uint16_t *vbase = scalar_ptr(v + (size_t)kvh * HD);
+    const int t_begin = split * tiles_per_split;
+    const int nt = min((seq_k + BN - 1) / BN - t_begin, tiles_per_split);      /* >= 1: the launcher makes no empty range */
+
+    /* LDS read offsets (elements from the start of the LDS; stage 1 of either tensor is TILE further).
+     * K operand (key block mb, k-step ks): row 16 mb + li, chunk 4 ks + lg = 16 (ks / 4) + (4 (ks % 4) + lg); the
+     * swizzle touches the low four bits of the chunk only, so four registers and immediate offsets do.
+     * V^T operand (dim block db of 16): transposing read of a 4-key x 16-dim block per 16-lane group, row 4 lg + li / 4
+     * (+ 16 for the second half of the keys), chunk 2 db + (li % 4) / 2 = 16 (db / 8) + (2 (db % 8) + ..). */
+    int k_rd[4], v_rd[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) k_rd[i] = li * HD + 8 * ((4 * i + lg) ^ swz(li));
+    {
+        const int vrow = 4 * lg + (li >> 2);
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            v_rd[i] = 2 * TILE + vrow * HD + 8 * ((2 * i + ((li & 3) >> 1)) ^ swz(vrow)) + 4 * (li & 1);
+    }
+
+    /* One tile row (1 KB) per instruction: lane i fills slot i of row r = 8 wave + j of the stage, i.e. fetches chunk
+     * i ^ swz(r) = i ^ 2 j. Tiles past the end of the range repeat its last tile and rows past seq_k the last row (their
+     * scores are masked). */
+    const uint32_t lane_b = 16u * (uint32_t)lane;
+    auto request_row = [&](const uint16_t *base, int tile, uint16_t *stage, int j) INLINE {
+        const int k0 = (t_begin + min(tile, nt - 1)) * BN;
+        const int row = min(k0 + 8 * wave + j, seq_k - 1);
+        const uint16_t *src = base + (size_t)row * ldi;
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(stage + (8 * wave + j) * HD));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     ::"s"(dst), "v"(lane_b ^ (32u * (uint32_t)j)), "s"(src) : "memory", "m0");
+    };
+
+    f32x4 o[32][2];                                  /* O^T: dims 16 db + 4 lg + r of query block nb */
+    float m_run[2], neg_m[2], bound[2];
+    f32x4 l_acc[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+#pragma unroll
+        for (int db = 0; db < 32; db++) {
+            o[db][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            asm volatile("" : "+a"(o[db][nb]));
+        }
+        m_run[nb] = -INFINITY; neg_m[nb] = 0.0f; bound[nb] = -INFINITY;
+        l_acc[nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    const float inv_scale_log2 = 1.0f / scale_log2;
+    /* The all-ones A operand of the row-sum product stays in four registers for the whole kernel (the empty asm hides
+     * the constant from the compiler): written afresh in front of the product, a move would be followed at once by
+     * an asm statement that reads its result, and the compiler places the wait states a matrix instruction needs
+     * behind an ordinary one only for matrix instructions it issues itself. */
+    u32x4 ones = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+    asm volatile("" : "+v"(ones));
+
+    /* ---- prologue: tile 0 of both tensors and K of tile 1, then Q ---- */
+#pragma unroll
+    for (int j = 0; j < 8; j++) request_row(kbase, 0, lds, j);
+#pragma unroll
+    for (int j = 0; j < 8; j++) request_row(vbase, 0, lds + 2 * TILE, j);
+#pragma unroll
+    for (int j = 0; j < 8; j++) request_row(kbase, 1, lds + TILE, j);
+
+    /* Q^T as B operands: for query block nb and k-step ks the lane holds dims 32 ks + 8 lg .. +7 of query 16 nb + li */
+    bf16x8 qb[2][16];
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+        const uint16_t *qp = q + (size_t)min(qrow0 + 16 * nb, seq_q - 1) * ldi + (size_t)head * HD + 8 * lg;
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++)
+            qb[nb][ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 32 * ks));
+    }
+    /* the tile requests are invisible to the compiler's wait-count bookkeeping: complete the loads it knows about
+     * here, so that it places no wait for them inside the loop (which would wait for the newest tile requests) */
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++) {
+            u32x4 t = __builtin_bit_cast(u32x4, qb[nb][ks]);
+            asm volatile("" : "+v"(t));
+            qb[nb][ks] = __builtin_bit_cast(bf16x8, t);
+        }
+    wait_vmcnt<0>();
+    lds_barrier();
+
+    /* ---- S^T = K Q^T of one tile: 2 key blocks x 2 query blocks, 16 k-steps of 32 dims; the operands of step
+     * ks + 1 are requested before the products of step ks; between(ks) is issued there too ---- */
+    f32x4 s[2][2];
+    auto scores = [&](int kstage, auto &&between) INLINE {
+        const uint16_t *kst = lds + kstage * TILE;
+        u32x4 ka[2][2];
+        auto read_k = [&](int ks) INLINE {
+#pragma unroll
+            for (int mb = 0; mb < 2; mb++)
+                ka[ks & 1][mb] = *reinterpret_cast<const u32x4 *>(&kst[k_rd[ks & 3] + 128 * (ks >> 2) + 16 * mb * HD]);
+        };
+        read_k(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++) {
+            if (ks < 15) read_k(ks + 1);
+            between(ks);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                for (int nb = 0; nb < 2; nb++) {
+                    if (ks == 0) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=&v"(s[mb][nb]) : "v"(ka[0][mb]), "v"(qb[nb][0]));
+                    else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(s[mb][nb]) : "v"(ka[ks & 1][mb]), "v"(qb[nb][ks]));
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    /* ---- online softmax of the scores in s (tile `tile` of the range) -> P^T as B operands in pw. The lane holds 8
+     * of the 32 scores of each of its two queries: keys 16 mb + 4 lg + r. The running max is only raised when some
+     * score of the wave exceeds it by more than 2^8; that test needs no cross-lane traffic (the four lanes of a
+     * query share the bound). ---- */
+    u32x4 pw[2];
+    auto softmax = [&](int tile) INLINE {
+        const int k0 = (t_begin + tile) * BN;
+        if (k0 + BN > seq_k) {                       /* the last tile of the sequence, partly filled */
+            const unsigned mine = ((1u << (seq_k - k0)) - 1u) >> (4 * lg);
+#pragma unroll
+            for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (!((mine >> (16 * mb + r)) & 1u)) {
+#pragma unroll
+                        for (int nb = 0; nb < 2; nb++) s[mb][nb][r] = -INFINITY;
+                    }
+        }
+        float lane_max[2];
+        bool raise = false;
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
+            const float a = max3(s[0][nb][0], s[0][nb][1], s[0][nb][2]);
+            const float b = max3(s[0][nb][3], s[1][nb][0], s[1][nb][1]);
+            const float c = max3(s[1][nb][2], s[1][nb][3], a);
+            lane_max[nb] = fmaxf(b, c);
+            raise = raise || lane_max[nb] > bound[nb];
+        }
+        if (__any(raise)) {
+            /* the accumulators are read by ordinary instructions here, perhaps right behind the products of the values:
+             * these have to leave the matrix core first (volatile asm statements keep their order, and the empty ones
+             * below make every read of an accumulator come after this one) */
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++) {
+                const float m_new = fmaxf(m_run[nb], quad_group_max(lane_max[nb]) * scale_log2);
+                const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - (m_new == -INFINITY ? 0.0f : m_new));
+                m_run[nb] = m_new;
+                neg_m[nb] = m_new == -INFINITY ? 0.0f : -m_new;
+                bound[nb] = (m_new + RESCALE_THRESHOLD) * inv_scale_log2;
+                l_acc[nb] *= alpha;
+#pragma unroll
+                for (int db = 0; db < 32; db++) {
+                    asm volatile("" : "+a"(o[db][nb]));
+                    f32x4 t = o[db][nb];
+                    t *= alpha;
+                    o[db][nb] = t;
+                    asm volatile("" : "+a"(o[db][nb]));
+                }
+            }
+        }
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
+            float p[8];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                p[r] = __builtin_amdgcn_exp2f(fmaf(s[0][nb][r], scale_log2, neg_m[nb]));
+                p[4 + r] = __builtin_amdgcn_exp2f(fmaf(s[1][nb][r], scale_log2, neg_m[nb]));
+            }
+            pw[nb] = u32x4{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
+        }
+    };
+
+    /* ---- O^T += V^T P^T of one tile: one k-step of 32 keys x 32 dim blocks x 2 query blocks, the V^T operands of
+     * the next two dim blocks requested before the products of these two ---- */
+    auto values = [&](int vstage) INLINE {
+        const uint16_t *vst = lds + vstage * TILE;            /* v_rd already points into V stage 0 */
+        s16x4 lo[2][2], hi[2][2];
+        auto read_v = [&](int g) INLINE {
+#pragma unroll
+            for (int d = 0; d < 2; d++) {
+                const int db = 2 * g + d;
+                const uint16_t *vp = &vst[v_rd[db & 7] + 128 * (db >> 3)];
+                lo[g & 1][d] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp));
+                hi[g & 1][d] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 16 * HD));
+            }
+        };
+        read_v(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++)
+            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(l_acc[nb]) : "v"(ones), "v"(pw[nb]));
+#pragma unroll
+        for (int g = 0; g < 16; g++) {
+            if (g < 15) read_v(g + 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int d = 0; d < 2; d++) {
+                const s16x8 both = __builtin_shufflevector(lo[g & 1][d], hi[g & 1][d], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                for (int nb = 0; nb < 2; nb++)
+                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(o[2 * g + d][nb]) : "v"(both), "v"(pw[nb]));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    /* the skew: scores and probabilities of tile 0. The products are asm statements, which the compiler's hazard
+     * bookkeeping does not see: a product's result must have left the matrix core before other instructions read it.
+     * In the loop the 66 products of the values stand between the last score product and the softmax that reads the
+     * scores; here idle cycles do. */
+    scores(0, [](int) INLINE {});
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]));
+    softmax(0);
+    lds_barrier();                                   /* K stage 0 has no readers any more */
+
+    /* Turn t (par = t % 2): K of tile t + 2 -> K stage par and V of tile t + 1 -> V stage par ^ 1 are requested, one
+     * row per k-step of the score product of tile t + 1 (K stage par ^ 1); then the values of tile t (V stage par,
+     * probabilities from the turn before) and the probabilities of tile t + 1. */
+    auto turn = [&](int t, int par) INLINE {
+        scores(par ^ 1, [&](int ks) INLINE {
+            if (ks < 8) request_row(kbase, t + 2, lds + par * TILE, ks);
+            else request_row(vbase, t + 1, lds + (2 + (par ^ 1)) * TILE, ks - 8);
+        });
+        values(par);
+        if (t + 1 < nt) softmax(t + 1);
+        wait_vmcnt<0>();
+        lds_barrier();
+    };
+    for (int t = 0; t < nt; t += 2) {
+        turn(t, 0);
+        if (t + 1 < nt) turn(t + 1, 1);
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");      /* the last products have left the matrix core */
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+#pragma unroll
+        for (int db = 0; db < 32; db++) asm volatile("" : "+a"(o[db][nb]));
+        asm volatile("" : "+v"(l_acc[nb]));
+    }
+
+    /* ---- the lane holds dims 16 db + 4 lg + {0..3} of its two queries ---- */
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+        const float l_tot = l_acc[nb][0];              /* every row of the ones product is the full sum */
+        const int qrow = qrow0 + 16 * nb;
+        if (qrow >= seq_q) continue;
+        if (SPLIT) {
+            const size_t prow = ((size_t)split * heads + head) * seq_q + qrow;
+            float *po = part.o + prow * HD + 4 * lg;
+#pragma unroll
+            for (int db = 0; db < 32; db++) *reinterpret_cast<f32x4 *>(po + 16 * db) = o[db][nb];
+            if (lg == 0) *reinterpret_cast<f32x2 *>(part.ml + 2 * prow) = f32x2{m_run[nb], l_tot};
+        } else {
+            const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+            uint16_t *op = out + (size_t)qrow * ldo + (size_t)head * HD + 4 * lg;
+#pragma unroll
+            for (int db = 0; db < 32; db++) {
+                uint2 w;
+                w.x = pack_bf16(o[db][nb][0] * inv, o[db][nb][1] * inv);
+                w.y = pack_bf16(o[db][nb][2] * inv, o[db][nb][3] * inv);
+                *reinterpret_cast<uint2 *>(op + 16 * db) = w;
+            }
+        }
+    }
+}
+
+#pragma clang diagnostic pop
+
+/* Combines the key ranges of a query: out = sum_r 2^(m_r - m) o_r / sum_r 2^(m_r - m) l_r with m the largest of the
+ * maxima. 64 threads per query row, 8 dims each. */
+__global__ void __launch_bounds__(256)
+k_fa_hd512_merge(uint16_t *__restrict__ out, int ldo, Partials part, int seq_q, int heads, int splits) {
+    const size_t rows = (size_t)heads * seq_q;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);       /* head * seq_q + query */
+    if (row >= rows) return;
+    const int t = threadIdx.x & 63;
+    float m = -INFINITY;
+    for (int r = 0; r < splits; r++) m = fmaxf(m, part.ml[2 * (r * rows + row)]);
+    float l = 0.0f, acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    for (int r = 0; r < splits; r++) {
+        const f32x2 ml = *reinterpret_cast<const f32x2 *>(part.ml + 2 * (r * rows + row));
+        const float w = ml[0] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ml[0] - m);
+        l += w * ml[1];
+        const float *po = part.o + (r * rows + row) * HD + 8 * t;
+        const f32x4 a = *reinterpret_cast<const f32x4 *>(po), b = *reinterpret_cast<const f32x4 *>(po + 4);
+#pragma unroll
+        for (int i = 0; i < 4; i++) { acc[i] += w * a[i]; acc[4 + i] += w * b[i]; }
+    }
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    const size_t head = row / seq_q, qrow = row - head * seq_q;
+    uint16_t *op = out + qrow * ldo + head * HD + 8 * t;                  /* output rows are 8-byte aligned, not more */
+    *reinterpret_cast<uint2 *>(op) = make_uint2(pack_bf16(acc[0] * inv, acc[1] * inv), pack_bf16(acc[2] * inv, acc[3] * inv));
+    *reinterpret_cast<uint2 *>(op + 4) = make_uint2(pack_bf16(acc[4] * inv, acc[5] * inv), pack_bf16(acc[6] * inv, acc[7] * inv));
+}
+
+int cu_count() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount >= 8)
+            n = prop.multiProcessorCount;
+        else {
+            (void)hipGetLastError();
+            n = 256;
+        }
+    }
+    return n;
+}
+
+}  // namespace
+
+/* How many key ranges a call is cut into, and the scratch it then needs (0 for one range). A turn of 32 keys takes a
+ * workgroup about 1 us, a round of workgroups over the CUs costs its turns plus about 8 us of start and end, and the
+ * merge reads and writes its partials at about 3 TB/s behind a launch. Host arithmetic only. */
+extern "C" size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int *splits_out) {
+    const long cus = cu_count();
+    const long tiles = (seq_k + BN - 1) / BN, wgs = (long)((seq_q + BM - 1) / BM) * heads;
+    const double rows_mb = (double)seq_q * heads * HD * 4 / 1e6;          /* one range's partial O, MB */
+    double best = 0.0;
+    int best_s = 1;
+    for (int s = 1; s <= 8 && s <= tiles; s++) {
+        const long per = (tiles + s - 1) / s, ranges = (tiles + per - 1) / per;
+        if (ranges != s) continue;
+        const long rounds = (wgs * ranges + cus - 1) / cus;
+        double us = rounds * (per * 1.0 + 8.0);
+        if (ranges > 1) us += 6.0 + 2.0 * ranges * rows_mb / 3.0;          /* MB / (TB/s) = us */
+        if (s == 1 || us < best * 0.97) { best = us; best_s = s; }
+    }
+    *splits_out = best_s;
+    if (best_s == 1) return 0;
+    const size_t rows = (size_t)seq_q * heads * best_s;
+    return rows * HD * sizeof(float) + rows * 2 * sizeof(float);
+}
+
+/* head_dim 512, no mask, not causal; rows 16-byte aligned (ldi % 8 == 0, ldo % 4 == 0), seq_k >= 1, scale > 0.
+ * `splits` and `scratch` as iris_hip_fa_hd512_plan says for the same sizes (scratch may be null for one range). */
+extern "C" int iris_hip_fa_hd512(void *stream, uint16_t *out, int ldo, const uint16_t *q,
+                                 const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
+                                 int seq_k, int heads, int kv_heads, float scale, int splits, void *scratch) {
+    hipStream_t st = (hipStream_t)stream;
+    const int tiles = (seq_k + BN - 1) / BN;
+    if (splits < 1 || splits > tiles || (splits > 1 && !scratch)) return (int)hipErrorInvalidValue;
+    const int per = (tiles + splits - 1) / splits;
+    if ((tiles + per - 1) / per != splits) return (int)hipErrorInvalidValue;      /* an empty range */
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd512<false>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd512<true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        configured = true;
+    }
+    const int q_tiles = (seq_q + BM - 1) / BM;
+    const int total = q_tiles * heads * splits;
+    const int per_xcd = (total + XCDS - 1) / XCDS;
+    const size_t rows = (size_t)seq_q * heads * splits;
+    Partials part = {reinterpret_cast<float *>(scratch), reinterpret_cast<float *>(scratch) + rows * HD};
+    const float scale_log2 = scale * 1.4426950408889634f;
+    if (splits == 1) {
+        hipLaunchKernelGGL((k_fa_fwd_hd512<false>), dim3(per_xcd * XCDS), dim3(THREADS), LDS_BYTES, st, out, ldo, q, k, v,
+                           ldi, seq_q, seq_k, heads, q_tiles, 1, per, total, per_xcd, heads / kv_heads, scale_log2, part);
+        return (int)hipGetLastError();
+    }
+    hipLaunchKernelGGL((k_fa_fwd_hd512<true>), dim3(per_xcd * XCDS), dim3(THREADS), LDS_BYTES, st, out, ldo, q, k, v,
+                       ldi, seq_q, seq_k, heads, q_tiles, splits, per, total, per_xcd, heads / kv_heads, scale_log2, part);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    const size_t merge_rows = (size_t)seq_q * heads;
+    hipLaunchKernelGGL(k_fa_hd512_merge, dim3((unsigned)((merge_rows + 3) / 4)), dim3(256), 0, st, out, ldo, part, seq_q,
+                       heads, splits);
+    return (int)hipGetLastError();
+}

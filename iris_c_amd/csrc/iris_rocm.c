@@ -41,6 +41,9 @@ static size_t g_q_scratch_bytes = 0;
 /* padded, aligned copy of q | k | v (and the padded output) for attention calls on other head sizes or alignments */
 static uint16_t *g_pack = NULL;
 static size_t g_pack_bytes = 0;
+/* partial results of the key ranges of a head_dim-512 attention call (f32 rows, maxima and sums) */
+static void *g_split = NULL;
+static size_t g_split_bytes = 0;
 #ifndef IRIS_DEV_PATH_ONLY
 /* staging buffer of the rotary tables being expanded: column map, row offsets, dictionary */
 static void *g_rope_stage = NULL;
@@ -113,8 +116,11 @@ void iris_dev_cleanup(void) {
     if (g_rope_stage) check(hipFree(g_rope_stage), "free");
     if (g_q_scratch) check(hipFree(g_q_scratch), "free");
     if (g_pack) check(hipFree(g_pack), "free");
+    if (g_split) check(hipFree(g_split), "free");
     g_pack = NULL;
     g_pack_bytes = 0;
+    g_split = NULL;
+    g_split_bytes = 0;
     g_q_scratch = NULL;
     g_q_scratch_bytes = 0;
     iris_lt_release();
@@ -184,10 +190,13 @@ void iris_dev_path_detach(void) {
     check(hipStreamSynchronize(g_stream), "sync");
     if (g_q_scratch) check(hipFree(g_q_scratch), "free");
     if (g_pack) check(hipFree(g_pack), "free");
+    if (g_split) check(hipFree(g_split), "free");
     g_q_scratch = NULL;
     g_q_scratch_bytes = 0;
     g_pack = NULL;
     g_pack_bytes = 0;
+    g_split = NULL;
+    g_split_bytes = 0;
     g_stream = NULL;
     g_ready = 0;
 }
@@ -297,6 +306,25 @@ void iris_dev_head_norm_rope_qk_streams(uint16_t *xq, uint16_t *xk, int ld,
                       split_half);
 }
 
+/* head_dim 256 / 512 on the matrix cores (rows 16-byte aligned). 512 without mask or causal limit, the VAE's call,
+ * takes the kernel in which a wave owns 32 whole queries; its key ranges, if it cuts any, leave their partial results
+ * in private scratch. Everything else takes the kernel that slices the head dim over the waves. Returns 0 or a HIP
+ * error; -1 when the scratch could not be had (already reported). */
+static int attention_wide(const char *what, const char *name512, const char *name_sliced, uint16_t *out, int ldo,
+                          const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi, int seq_q, int seq_k,
+                          int heads, int kv_heads, int head_dim, float scale, int causal, const int *key_mask) {
+    if (head_dim == 512 && !causal && !key_mask) {
+        int splits = 1;
+        const size_t need = iris_hip_fa_hd512_plan(seq_q, seq_k, heads, &splits);
+        if (need && !scratch_fit(&g_split, &g_split_bytes, need, what)) return -1;
+        g_last_kernel = name512;
+        return iris_hip_fa_hd512(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, splits, g_split);
+    }
+    g_last_kernel = name_sliced;
+    return iris_hip_fa_sliced(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, head_dim, scale, causal != 0,
+                              key_mask);
+}
+
 /* wq == NULL: plain attention. Otherwise Q is normalised and rotated on the way in. */
 static void attention(const char *what, uint16_t *out, int ldo,
                       const uint16_t *q, const uint16_t *k, const uint16_t *v,
@@ -346,9 +374,9 @@ static void attention(const char *what, uint16_t *out, int ldo,
     }
     const int mfma_args = seq_k > 0 && scale > 0.0f && head_dim <= 512 && (!key_mask || seq_k <= IRIS_FA_MAX_MASKED_KEYS);
     if (mfma_ok && !wq && (head_dim == 256 || head_dim == 512)) {
-        g_last_kernel = "fa_sliced";
-        err = iris_hip_fa_sliced(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads,
-                                 head_dim, scale, causal != 0, key_mask);
+        err = attention_wide(what, "fa_hd512", "fa_sliced", out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, head_dim,
+                             scale, causal, key_mask);
+        if (err < 0) return;
     } else if (mfma_args) {
         /* Any head_dim <= 512, any stride and alignment: q | k | v copied into one fused row buffer with
          * every head padded with zeros to the next of 128 / 256 / 512 dims, the matrix-core kernel of that
@@ -369,9 +397,10 @@ static void attention(const char *what, uint16_t *out, int ldo,
                 err = iris_hip_fa_hd128(g_stream, outp, ldout, packed, pk, pv, ldp, seq_q, seq_k, heads, kv_heads,
                                         scale, causal != 0, key_mask);
             } else {
-                g_last_kernel = wq ? "fa_sliced_packed_qnorm" : "fa_sliced_packed";
-                err = iris_hip_fa_sliced(g_stream, outp, ldout, packed, pk, pv, ldp, seq_q, seq_k, heads, kv_heads,
-                                         hdp, scale, causal != 0, key_mask);
+                err = attention_wide(what, wq ? "fa_hd512_packed_qnorm" : "fa_hd512_packed",
+                                     wq ? "fa_sliced_packed_qnorm" : "fa_sliced_packed", outp, ldout, packed, pk, pv, ldp,
+                                     seq_q, seq_k, heads, kv_heads, hdp, scale, causal, key_mask);
+                if (err < 0) return;
             }
         }
         if (!err && !direct_out)

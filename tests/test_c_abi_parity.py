@@ -34,7 +34,7 @@ def test_c_program_parity_on_gpu():
     r = _run()
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert "all checks passed" in r.stdout and "kernel: fa_sliced" in r.stdout
+    assert "all checks passed" in r.stdout and "kernel: fa_hd512" in r.stdout
 
 
 @pytest.mark.gpu

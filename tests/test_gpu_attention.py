@@ -370,8 +370,9 @@ def test_output_stride_and_interior_pointers(dev, orc, fa):
 @pytest.mark.parametrize("hd,heads,kv", [(512, 1, 1), (512, 2, 1), (256, 3, 3), (256, 4, 2)])
 @pytest.mark.parametrize("seq_q,seq_k,causal,masked", [(150, 150, False, False), (1, 1, False, False), (33, 95, False, True),
                                                          (64, 64, True, False), (257, 257, True, True), (130, 1000, False, False)])
-def test_sliced_kernel_head_dims_256_512(dev, orc, hd, heads, kv, seq_q, seq_k, causal, masked):
-    """head_dim 256 / 512 (the VAE's single 512-wide head) run on the matrix cores too."""
+def test_wide_heads_256_512(dev, orc, hd, heads, kv, seq_q, seq_k, causal, masked):
+    """head_dim 256 / 512 run on the matrix cores too: 512 without mask or causal limit (the VAE's single 512-wide
+    head) in the kernel whose waves own whole queries, the rest in the kernel that slices the head dim over the waves."""
     buf, ldi = random_case(hd + heads + seq_q, seq_q, seq_k, heads, kv, hd=hd)
     qd, kd = heads * hd, kv * hd
     mask = None
@@ -380,9 +381,9 @@ def test_sliced_kernel_head_dims_256_512(dev, orc, hd, heads, kv, seq_q, seq_k, 
         mask[0] = 1                                        # every causal row keeps a valid key
     scale = float(1 / np.sqrt(hd))
     out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
-    assert kernel == "fa_sliced"
+    assert kernel == ("fa_hd512" if hd == 512 and not causal and not masked else "fa_sliced")
     want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
-    assert_close(O.bf16_to_f32(out[:seq_q]), want, f"sliced hd={hd} {seq_q}x{seq_k}")
+    assert_close(O.bf16_to_f32(out[:seq_q]), want, f"wide hd={hd} {seq_q}x{seq_k}")
 
 
 def test_vae_shape_full_size_sampled_rows(dev, orc):
@@ -392,7 +393,7 @@ def test_vae_shape_full_size_sampled_rows(dev, orc):
     buf, ldi = random_case(77, seq, seq, 1, 1, hd=hd)
     scale = float(1 / np.sqrt(hd))
     out, kernel = dev.attention(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale)
-    assert kernel == "fa_sliced"
+    assert kernel == "fa_hd512"
     rows = sample_rows(seq, n=20)
     want = orc.attention_bf16(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale, rows=rows)
     assert_close(O.bf16_to_f32(out)[rows], want, "VAE shape sampled")
@@ -410,8 +411,8 @@ def test_vae_shape_at_its_largest_50176_tokens(dev, orc):
     buf, ldi = random_case(78, seq, seq, 1, 1, hd=hd)
     scale = float(1 / np.sqrt(hd))
     out, kernel = dev.attention(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale)
-    assert kernel == "fa_sliced"
-    rows = np.unique(np.r_[sample_rows(seq, n=10), [63, 64, 25087, 25088, seq - 65, seq - 64]]).astype(np.int32)
+    assert kernel == "fa_hd512"
+    rows = np.unique(np.r_[sample_rows(seq, n=10), [127, 128, 25087, 25088, seq - 129, seq - 128]]).astype(np.int32)
     want = orc.attention_bf16(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale, rows=rows)
     assert_close(O.bf16_to_f32(out[rows]), want, "VAE 50176 tokens sampled")
     buf[:, 2 * hd:] = buf[5, 2 * hd:]
@@ -452,7 +453,8 @@ def test_other_head_dims_run_on_the_matrix_cores_through_a_padded_copy(dev, orc,
     scale = 1 / np.sqrt(hd)
     ldo = heads * hd + 3
     out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq, seq, heads, kv, hd, scale, causal, mask, ldo=ldo)
-    assert kernel == ("fa_hd128_packed" if hd <= 128 else "fa_sliced_packed")
+    wide = "fa_hd512_packed" if hd > 256 and not causal and not masked else "fa_sliced_packed"
+    assert kernel == ("fa_hd128_packed" if hd <= 128 else wide)
     want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq, seq, heads, kv, hd, scale, causal, mask)
     assert_close(O.bf16_to_f32(out[:, :heads * hd]), want, f"padded copy hd={hd}")
     assert np.all(out[:, heads * hd:] == 0x7fc0)              # nothing written past the head columns
@@ -466,7 +468,7 @@ def test_misaligned_rows_run_on_the_matrix_cores_through_an_aligned_copy(dev, or
     qd = heads * hd
     scale = float(1 / np.sqrt(hd))
     out, kernel = dev.attention(buf, ldi, qoff, qoff + qd, qoff + 2 * qd, seq, seq, heads, heads, hd, scale)
-    assert kernel == ("fa_hd128_packed" if hd == 128 else "fa_sliced_packed")
+    assert kernel == {128: "fa_hd128_packed", 256: "fa_sliced_packed", 512: "fa_hd512_packed"}[hd]
     want = orc.attention_bf16(buf, ldi, qoff, qoff + qd, qoff + 2 * qd, seq, seq, heads, heads, hd, scale)
     assert_close(O.bf16_to_f32(out), want, f"misaligned hd={hd} pad={pad} offset={qoff}")
 

@@ -224,7 +224,7 @@ def test_vae_resblock_and_attention_chain(dev, orc):
     lib.iris_dev_conv2d(t2b, t1b, d["qkvw"], d["qkvb"], hw, 1, c, 3 * c, 1, 1, 0, 0)
     lib.iris_dev_f32_to_bf16(qkvd, t2b, hw * 3 * c)
     lib.iris_dev_attention(od, c, qkvd, ptr_add(qkvd, 2 * c), ptr_add(qkvd, 4 * c), 3 * c, hw, hw, 1, 1, c, float(1 / np.sqrt(c)), 0, None)
-    assert dev.dev.last_kernel() == "fa_sliced"
+    assert dev.dev.last_kernel() == "fa_hd512"
     lib.iris_dev_linear_f32(outb, od, d["ow"], hw, c, c)
     lib.iris_dev_add_bias(outb, d["ob"], hw, c)
     lib.iris_dev_add(outb, d["xa"], hw * c)
