@@ -55,7 +55,7 @@ constexpr int BM = 128;             /* queries per workgroup */
 constexpr int THREADS = 256;
 constexpr int TILE = BN * HD;       /* elements of a K (or V) tile: 32 KB */
 constexpr int XCDS = 8;
-constexpr size_t LDS_BYTES = 4 * (size_t)TILE * sizeof(uint16_t);
+constexpr size_t LDS_BYTES = 5 * (size_t)TILE * sizeof(uint16_t);      /* three K stages, two V stages: all 160 KB */
 constexpr float RESCALE_THRESHOLD = 8.0f;   /* log2 units */
 
 /* Every lambda below is inlined by the always-inline pass, before anything else runs: a closure that is only
@@ -124,32 +124,41 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     const int t_begin = split * tiles_per_split;
     const int nt = min((seq_k + BN - 1) / BN - t_begin, tiles_per_split);      /* >= 1: the launcher makes no empty range */
 
-    /* LDS read offsets (elements from the start of the LDS; stage 1 of either tensor is TILE further).
+    /* LDS: K stages 0, 1, 2 | V stages 0, 1 (TILE elements each). Read offsets in elements from the start of the LDS.
      * K operand (key block mb, k-step ks): row 16 mb + li, chunk 4 ks + lg = 16 (ks / 4) + (4 (ks % 4) + lg); the
-     * swizzle touches the low four bits of the chunk only, so four registers and immediate offsets do.
+     * swizzle touches the low four bits of the chunk only, so four registers and immediate offsets do; they run from
+     * K stage to K stage with the tiles.
      * V^T operand (dim block db of 16): transposing read of a 4-key x 16-dim block per 16-lane group, row 4 lg + li / 4
      * (+ 16 for the second half of the keys), chunk 2 db + (li % 4) / 2 = 16 (db / 8) + (2 (db % 8) + ..). */
-    int k_rd[4], v_rd[8];
+    int k_cur[4], v_rd[8];
 #pragma unroll
-    for (int i = 0; i < 4; i++) k_rd[i] = li * HD + 8 * ((4 * i + lg) ^ swz(li));
+    for (int i = 0; i < 4; i++) k_cur[i] = li * HD + 8 * ((4 * i + lg) ^ swz(li));
     {
         const int vrow = 4 * lg + (li >> 2);
 #pragma unroll
         for (int i = 0; i < 8; i++)
-            v_rd[i] = 2 * TILE + vrow * HD + 8 * ((2 * i + ((li & 3) >> 1)) ^ swz(vrow)) + 4 * (li & 1);
+            v_rd[i] = 3 * TILE + vrow * HD + 8 * ((2 * i + ((li & 3) >> 1)) ^ swz(vrow)) + 4 * (li & 1);
     }
 
     /* One tile row (1 KB) per instruction: lane i fills slot i of row r = 8 wave + j of the stage, i.e. fetches chunk
-     * i ^ swz(r) = i ^ 2 j. Tiles past the end of the range repeat its last tile and rows past seq_k the last row (their
-     * scores are masked). */
-    const uint32_t lane_b = 16u * (uint32_t)lane;
-    auto request_row = [&](const uint16_t *base, int tile, uint16_t *stage, int j) INLINE {
-        const int k0 = (t_begin + min(tile, nt - 1)) * BN;
-        const int row = min(k0 + 8 * wave + j, seq_k - 1);
-        const uint16_t *src = base + (size_t)row * ldi;
-        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(stage + (8 * wave + j) * HD));
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                     ::"s"(dst), "v"(lane_b ^ (32u * (uint32_t)j)), "s"(src) : "memory", "m0");
+     * i ^ swz(r) = i ^ 2 j of global row r. A wave's eight rows of a tile differ in the per-lane offset only (row j:
+     * j row strides further), kept in eight registers, so that a request is three instructions: M0, a wait state,
+     * the load, with one scalar source pointer per tile. A tile never reaches past the last key: the last tile of a
+     * sequence whose length is not a multiple of 32 is moved back to end with it, and the keys it then shares
+     * with the tile before are masked there (seq_k >= 32). Tiles past the end of the range repeat its last tile.
+     * `stage` counts TILEs from the start of the LDS. */
+    uint32_t lane_off[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) lane_off[j] = ((16u * (uint32_t)lane) ^ (32u * (uint32_t)j)) + (uint32_t)j * (uint32_t)ldi * 2u;
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds)) + (uint32_t)(8 * wave * HD * 2);
+    auto tile_rows = [&](const uint16_t *base, int tile) INLINE {          /* the wave's first row of a tile of the range */
+        const int k0 = min((t_begin + min(tile, nt - 1)) * BN, seq_k - BN);
+        return base + (size_t)(k0 + 8 * wave) * ldi;
+    };
+    auto request_row = [&](const uint16_t *rows, int stage, int j) INLINE {
+        const uint32_t dst = lds0 + (uint32_t)(stage * TILE * 2);
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
+                     ::"s"(dst), "n"(j * HD * 2), "v"(lane_off[j]), "s"(rows) : "memory", "m0", "scc");
     };
 
     f32x4 o[32][2];                                  /* O^T: dims 16 db + 4 lg + r of query block nb */
@@ -173,13 +182,18 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     u32x4 ones = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
     asm volatile("" : "+v"(ones));
 
-    /* ---- prologue: tile 0 of both tensors and K of tile 1, then Q ---- */
+    /* ---- prologue: K of tiles 0, 1, 2 and V of tile 0, then Q ---- */
+    {
+        const uint16_t *k0r = tile_rows(kbase, 0), *v0r = tile_rows(vbase, 0), *k1r = tile_rows(kbase, 1), *k2r = tile_rows(kbase, 2);
 #pragma unroll
-    for (int j = 0; j < 8; j++) request_row(kbase, 0, lds, j);
+        for (int j = 0; j < 8; j++) request_row(k0r, 0, j);
 #pragma unroll
-    for (int j = 0; j < 8; j++) request_row(vbase, 0, lds + 2 * TILE, j);
+        for (int j = 0; j < 8; j++) request_row(v0r, 3, j);
 #pragma unroll
-    for (int j = 0; j < 8; j++) request_row(kbase, 1, lds + TILE, j);
+        for (int j = 0; j < 8; j++) request_row(k1r, 1, j);
+#pragma unroll
+        for (int j = 0; j < 8; j++) request_row(k2r, 2, j);
+    }
 
     /* Q^T as B operands: for query block nb and k-step ks the lane holds dims 32 ks + 8 lg .. +7 of query 16 nb + li */
     bf16x8 qb[2][16];
@@ -203,32 +217,33 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     wait_vmcnt<0>();
     lds_barrier();
 
-    /* ---- S^T = K Q^T of one tile: 2 key blocks x 2 query blocks, 16 k-steps of 32 dims; the operands of step
-     * ks + 1 are requested before the products of step ks; between(ks) is issued there too ---- */
+    /* ---- S^T = K Q^T of one tile into s: 2 key blocks x 2 query blocks, 16 k-steps of 32 dims. A wave that is
+     * alone on its SIMD issues in order, and what it issues between two products runs while the matrix core works on
+     * the first: one memory instruction per gap is free, more are not. So the two operand reads of k-step ks + KD
+     * stand behind the first and the third product of k-step ks, and between(i) behind the i-th of the 64 products
+     * is where the caller puts its tile requests. ---- */
+    constexpr int KD = 2;
     f32x4 s[2][2];
-    auto scores = [&](int kstage, auto &&between) INLINE {
-        const uint16_t *kst = lds + kstage * TILE;
-        u32x4 ka[2][2];
-        auto read_k = [&](int ks) INLINE {
-#pragma unroll
-            for (int mb = 0; mb < 2; mb++)
-                ka[ks & 1][mb] = *reinterpret_cast<const u32x4 *>(&kst[k_rd[ks & 3] + 128 * (ks >> 2) + 16 * mb * HD]);
+    auto scores = [&](auto &&between) INLINE {
+        u32x4 ka[KD + 1][2];
+        auto read_k = [&](int ks, int mb) INLINE {
+            ka[ks % (KD + 1)][mb] = *reinterpret_cast<const u32x4 *>(&lds[k_cur[ks & 3] + 128 * (ks >> 2) + 16 * mb * HD]);
         };
-        read_k(0);
+#pragma unroll
+        for (int ks = 0; ks < KD; ks++) { read_k(ks, 0); read_k(ks, 1); }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ks = 0; ks < 16; ks++) {
-            if (ks < 15) read_k(ks + 1);
-            between(ks);
-            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int mb = 0; mb < 2; mb++)
 #pragma unroll
                 for (int nb = 0; nb < 2; nb++) {
                     if (ks == 0) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=&v"(s[mb][nb]) : "v"(ka[0][mb]), "v"(qb[nb][0]));
-                    else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(s[mb][nb]) : "v"(ka[ks & 1][mb]), "v"(qb[nb][ks]));
+                    else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(s[mb][nb]) : "v"(ka[ks % (KD + 1)][mb]), "v"(qb[nb][ks]));
+                    if (nb == 0 && ks + KD < 16) read_k(ks + KD, mb);
+                    between(4 * ks + 2 * mb + nb);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
@@ -239,8 +254,8 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     u32x4 pw[2];
     auto softmax = [&](int tile) INLINE {
         const int k0 = (t_begin + tile) * BN;
-        if (k0 + BN > seq_k) {                       /* the last tile of the sequence, partly filled */
-            const unsigned mine = ((1u << (seq_k - k0)) - 1u) >> (4 * lg);
+        if (k0 + BN > seq_k) {                       /* the last tile of the sequence: moved back by k0 + 32 - seq_k keys, which are masked */
+            const unsigned mine = (~0u << (k0 + BN - seq_k)) >> (4 * lg);
 #pragma unroll
             for (int mb = 0; mb < 2; mb++)
 #pragma unroll
@@ -261,8 +276,8 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             raise = raise || lane_max[nb] > bound[nb];
         }
         if (__any(raise)) {
-            /* the accumulators are read by ordinary instructions here, perhaps right behind the products of the values:
-             * these have to leave the matrix core first (volatile asm statements keep their order, and the empty ones
+            /* the accumulators are read by ordinary instructions here, right behind the products of the values: these
+             * have to leave the matrix core first (volatile asm statements keep their order, and the empty ones
              * below make every read of an accumulator come after this one) */
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
@@ -272,6 +287,7 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                 m_run[nb] = m_new;
                 neg_m[nb] = m_new == -INFINITY ? 0.0f : -m_new;
                 bound[nb] = (m_new + RESCALE_THRESHOLD) * inv_scale_log2;
+                asm volatile("" : "+v"(l_acc[nb]));
                 l_acc[nb] *= alpha;
 #pragma unroll
                 for (int db = 0; db < 32; db++) {
@@ -295,66 +311,84 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         }
     };
 
-    /* ---- O^T += V^T P^T of one tile: one k-step of 32 keys x 32 dim blocks x 2 query blocks, the V^T operands of
-     * the next two dim blocks requested before the products of these two ---- */
-    auto values = [&](int vstage) INLINE {
+    /* ---- O^T += V^T P^T of one tile: one k-step of 32 keys x 32 dim blocks x 2 query blocks, in 16 groups of two
+     * dim blocks = four products; the four transposing reads of group g + VD stand one behind each product of
+     * group g, between(i) behind the i-th of the 64 products ---- */
+    constexpr int VD = 2;
+    auto values = [&](int vstage, auto &&between) INLINE {
         const uint16_t *vst = lds + vstage * TILE;            /* v_rd already points into V stage 0 */
-        s16x4 lo[2][2], hi[2][2];
-        auto read_v = [&](int g) INLINE {
-#pragma unroll
-            for (int d = 0; d < 2; d++) {
-                const int db = 2 * g + d;
-                const uint16_t *vp = &vst[v_rd[db & 7] + 128 * (db >> 3)];
-                lo[g & 1][d] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp));
-                hi[g & 1][d] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 16 * HD));
-            }
+        s16x4 lo[VD + 1][2], hi[VD + 1][2];
+        auto read_v = [&](int g, int r) INLINE {                /* r: dim block 2 g + r / 2, keys 0-15 or 16-31 of the tile */
+            const int db = 2 * g + (r >> 1);
+            const uint16_t *vp = &vst[v_rd[db & 7] + 128 * (db >> 3)];
+            if (r & 1) hi[g % (VD + 1)][r >> 1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp + 16 * HD));
+            else lo[g % (VD + 1)][r >> 1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp));
         };
-        read_v(0);
+#pragma unroll
+        for (int g = 0; g < VD; g++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) read_v(g, r);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int nb = 0; nb < 2; nb++)
             asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(l_acc[nb]) : "v"(ones), "v"(pw[nb]));
 #pragma unroll
         for (int g = 0; g < 16; g++) {
-            if (g < 15) read_v(g + 1);
-            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int d = 0; d < 2; d++) {
-                const s16x8 both = __builtin_shufflevector(lo[g & 1][d], hi[g & 1][d], 0, 1, 2, 3, 4, 5, 6, 7);
+                const s16x8 both = __builtin_shufflevector(lo[g % (VD + 1)][d], hi[g % (VD + 1)][d], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
-                for (int nb = 0; nb < 2; nb++)
+                for (int nb = 0; nb < 2; nb++) {
                     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(o[2 * g + d][nb]) : "v"(both), "v"(pw[nb]));
+                    if (g + VD < 16) read_v(g + VD, 2 * d + nb);
+                    between(4 * g + 2 * d + nb);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
-            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    /* the skew: scores and probabilities of tile 0. The products are asm statements, which the compiler's hazard
-     * bookkeeping does not see: a product's result must have left the matrix core before other instructions read it.
-     * In the loop the 66 products of the values stand between the last score product and the softmax that reads the
-     * scores; here idle cycles do. */
-    scores(0, [](int) INLINE {});
+    /* The scores run one tile ahead of the values: those of tile 0 here. The products are asm statements, which the
+     * compiler's hazard bookkeeping does not see: a product's result must have left the matrix core before other
+     * instructions read it. In the loop the products of the values stand between the last score product of a tile
+     * and the softmax that reads its scores; here idle cycles do. */
+    scores([](int) INLINE {});
     asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]));
     softmax(0);
     lds_barrier();                                   /* K stage 0 has no readers any more */
+    int kstage = 1;                                  /* where the K operand offsets point: the stage of tile t + 1 */
+#pragma unroll
+    for (int i = 0; i < 4; i++) k_cur[i] += TILE;
 
-    /* Turn t (par = t % 2): K of tile t + 2 -> K stage par and V of tile t + 1 -> V stage par ^ 1 are requested, one
-     * row per k-step of the score product of tile t + 1 (K stage par ^ 1); then the values of tile t (V stage par,
-     * probabilities from the turn before) and the probabilities of tile t + 1. */
+    /* Turn t (par = t % 2): score products of tile t + 1 (K stage (t + 1) % 3), value products of tile t (V stage par,
+     * probabilities from the turn before), softmax of tile t + 1. V of tile t + 1 -> V stage par ^ 1 is requested
+     * during the score products (its last readers were the value products of turn t - 1), K of tile t + 3 -> K stage
+     * t % 3 during the value products (last read by the score products of turn t - 1), one row every eighth
+     * product, so that the four waves keep the CU's one load path half busy all the time instead of saturating it
+     * for a part of the turn. At the end of the turn everything but the eight newest requests (K of tile t + 3) must
+     * have landed. */
     auto turn = [&](int t, int par) INLINE {
-        scores(par ^ 1, [&](int ks) INLINE {
-            if (ks < 8) request_row(kbase, t + 2, lds + par * TILE, ks);
-            else request_row(vbase, t + 1, lds + (2 + (par ^ 1)) * TILE, ks - 8);
+        const uint16_t *vrows = tile_rows(vbase, t + 1), *krows = tile_rows(kbase, t + 3);
+        scores([&](int i) INLINE {
+            if ((i & 7) == 5) request_row(vrows, 3 + (par ^ 1), i >> 3);
         });
-        values(par);
+        const int kreq = kstage == 0 ? 2 : kstage - 1;       /* t % 3 */
+        values(par, [&](int i) INLINE {
+            if ((i & 7) == 5) request_row(krows, kreq, i >> 3);
+        });
         if (t + 1 < nt) softmax(t + 1);
-        wait_vmcnt<0>();
+        const int step = kstage == 2 ? -2 * TILE : TILE;
+        kstage = kstage == 2 ? 0 : kstage + 1;
+#pragma unroll
+        for (int i = 0; i < 4; i++) k_cur[i] += step;
+        wait_vmcnt<8>();
         lds_barrier();
     };
     for (int t = 0; t < nt; t += 2) {
         turn(t, 0);
         if (t + 1 < nt) turn(t + 1, 1);
     }
+    wait_vmcnt<0>();                                  /* nothing may still be on its way into the LDS when it is given back */
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");      /* the last products have left the matrix core */
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
@@ -458,14 +492,14 @@ extern "C" size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int *s
     return rows * HD * sizeof(float) + rows * 2 * sizeof(float);
 }
 
-/* head_dim 512, no mask, not causal; rows 16-byte aligned (ldi % 8 == 0, ldo % 4 == 0), seq_k >= 1, scale > 0.
+/* head_dim 512, no mask, not causal; rows 16-byte aligned (ldi % 8 == 0, ldo % 4 == 0), seq_k >= 32, scale > 0.
  * `splits` and `scratch` as iris_hip_fa_hd512_plan says for the same sizes (scratch may be null for one range). */
 extern "C" int iris_hip_fa_hd512(void *stream, uint16_t *out, int ldo, const uint16_t *q,
                                  const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
                                  int seq_k, int heads, int kv_heads, float scale, int splits, void *scratch) {
     hipStream_t st = (hipStream_t)stream;
     const int tiles = (seq_k + BN - 1) / BN;
-    if (splits < 1 || splits > tiles || (splits > 1 && !scratch)) return (int)hipErrorInvalidValue;
+    if (seq_k < BN || splits < 1 || splits > tiles || (splits > 1 && !scratch)) return (int)hipErrorInvalidValue;
     const int per = (tiles + splits - 1) / splits;
     if ((tiles + per - 1) / per != splits) return (int)hipErrorInvalidValue;      /* an empty range */
     static bool configured = false;

@@ -73,8 +73,8 @@ int iris_hip_fa_sliced(void *stream, uint16_t *out, int ldo, const uint16_t *q,
 /* head_dim 512 without mask or causal limit (the VAE's call): one wave per SIMD owns 32 queries and all 512 output
  * dims; the keys may be cut into ranges that a second launch merges. iris_hip_fa_hd512_plan says how many ranges a
  * call of these sizes takes and returns the bytes of scratch it then needs (0 for one range; host arithmetic, no
- * GPU needed); iris_hip_fa_hd512 wants exactly that `splits` and a scratch of that size, 16-byte aligned. Same
- * argument conditions as iris_hip_fa_hd128 otherwise. */
+ * GPU needed); iris_hip_fa_hd512 wants exactly that `splits` and a scratch of that size, 16-byte aligned, and at
+ * least 32 keys. Same argument conditions as iris_hip_fa_hd128 otherwise. */
 size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int *splits);
 int iris_hip_fa_hd512(void *stream, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
                       const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads,

@@ -313,7 +313,7 @@ void iris_dev_head_norm_rope_qk_streams(uint16_t *xq, uint16_t *xk, int ld,
 static int attention_wide(const char *what, const char *name512, const char *name_sliced, uint16_t *out, int ldo,
                           const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi, int seq_q, int seq_k,
                           int heads, int kv_heads, int head_dim, float scale, int causal, const int *key_mask) {
-    if (head_dim == 512 && !causal && !key_mask) {
+    if (head_dim == 512 && !causal && !key_mask && seq_k >= 32) {          /* its key tiles are 32 whole rows */
         int splits = 1;
         const size_t need = iris_hip_fa_hd512_plan(seq_q, seq_k, heads, &splits);
         if (need && !scratch_fit(&g_split, &g_split_bytes, need, what)) return -1;
