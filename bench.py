@@ -939,6 +939,12 @@ def main():
                 entry.update(cpu_seconds=round(secs, 4), cpu_tflops=round(fl / secs / 1e12, 4), cpu_threads=threads,
                              cpu_query_chunk=chunk)
             shapes.append(entry)
+        # the VAE's mid-block attention of a 1024 x 1024 image: one head of 512 over 16384 tokens (no norm+rope in front)
+        v = only_one(dev, hip, stream, rng, "VAE", 20, args.settle_ms / 2)
+        shapes.append({"config": "VAE", "seq": 16384, "heads": 1, "kv_heads": 1, "head_dim": 512, "kernel": v["kernel"],
+                       "attention_ms": v["attention_ms_mean"], "attention_ms_median": v["attention_ms_median"],
+                       "attention_ms_min": v["attention_ms_min"], "attention_tflops": v["tflops"],
+                       "attention_frac_of_mfma_peak": round(v["tflops"] / PEAK_BF16_TFLOPS, 4)})
         out["shapes"] = shapes
 
     if not args.no_shapes:

@@ -469,9 +469,12 @@ int cu_count() {
 
 }  // namespace
 
-/* How many key ranges a call is cut into, and the scratch it then needs (0 for one range). A turn of 32 keys takes a
- * workgroup about 1 us, a round of workgroups over the CUs costs its turns plus about 8 us of start and end, and the
- * merge reads and writes its partials at about 3 TB/s behind a launch. Host arithmetic only. */
+/* How many key ranges a call is cut into, and the scratch it then needs (0 for one range). Host arithmetic only.
+ * Fitted to every number of ranges at 256 .. 50176 tokens: a turn of 32 keys takes a workgroup 1.6 us when all CUs
+ * are busy and 1.3 us when few are (the clock follows the load), a round of workgroups costs its turns plus about
+ * 8 us of start and end, and the merge reads and writes the partial rows at about 6 TB/s (they are still in the
+ * caches) behind a launch of 4 us and half a microsecond per range. The choice is within 3 % of the best count from
+ * 9216 tokens on and within 6 % below (where every count from 4 to 8 is within 10 % of every other). */
 extern "C" size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int *splits_out) {
     const long cus = cu_count();
     const long tiles = (seq_k + BN - 1) / BN, wgs = (long)((seq_q + BM - 1) / BM) * heads;
@@ -481,9 +484,10 @@ extern "C" size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int *s
     for (int s = 1; s <= 8 && s <= tiles; s++) {
         const long per = (tiles + s - 1) / s, ranges = (tiles + per - 1) / per;
         if (ranges != s) continue;
-        const long rounds = (wgs * ranges + cus - 1) / cus;
-        double us = rounds * (per * 1.0 + 8.0);
-        if (ranges > 1) us += 6.0 + 2.0 * ranges * rows_mb / 3.0;          /* MB / (TB/s) = us */
+        const long full = wgs * ranges / cus, rest = wgs * ranges % cus;
+        double us = full * (per * 1.6 + 8.0);
+        if (rest) us += per * (1.3 + 0.3 * (double)rest / cus) + 8.0;
+        if (ranges > 1) us += 4.0 + 0.5 * ranges + 2.0 * ranges * rows_mb / 6.0;          /* MB / (TB/s) = us */
         if (s == 1 || us < best * 0.97) { best = us; best_s = s; }
     }
     *splits_out = best_s;
