@@ -150,3 +150,34 @@ def test_double_stream_step_replayed_from_a_graph():
         assert np.array_equal(dev.get(out, (seq, case["ldo"]), np.uint16), want), f"replay {replay} differs from the eager step"
     g.rt.hipGraphExecDestroy(run)
     dev.free_all()
+
+
+def test_head_dim_512_attention_with_key_ranges_replayed_from_a_graph():
+    """The VAE's attention call at 4096 tokens: two launches (key ranges, then their merge through private scratch).
+    Once the scratch exists the call is captured; every replay, with eager calls of another size between them that
+    overwrite the same scratch, equals the eager result."""
+    import oracle as O
+    dev, g = Dev(), Graphs()
+    lib, stream = dev.lib, _vp(dev.lib.iris_dev_stream())
+    rng = np.random.default_rng(5)
+    seq, hd = 4096, 512
+    buf = O.f32_to_bf16(rng.standard_normal((seq, 3 * hd)).astype(np.float32))
+    rows, out, other = dev.put(buf), dev.alloc(seq * hd * 2), dev.alloc(seq * hd * 2)
+    scale = float(1 / np.sqrt(hd))
+    args = (out, hd, rows, ptr_add(rows, 2 * hd), ptr_add(rows, 4 * hd), 3 * hd, seq, seq, 1, 1, hd, scale, 0, None)
+    small = (other, hd, rows, ptr_add(rows, 2 * hd), ptr_add(rows, 4 * hd), 3 * hd, 1000, 1000, 1, 1, hd, scale, 0, None)
+    lib.iris_dev_attention(*args)                                   # outside: the scratch is sized
+    dev.check()
+    assert dev.dev.last_kernel() == "fa_hd512"
+    want = dev.get(out, (seq, hd), np.uint16)
+    run = g.capture(stream, lambda: lib.iris_dev_attention(*args))
+    dev.check()
+    for replay in range(3):
+        junk = np.full((seq, hd), 0x7fc0 + replay, np.uint16)
+        lib.iris_dev_upload(out, junk.ctypes.data_as(_vp), junk.nbytes)
+        lib.iris_dev_attention(*small)                              # eager work on the same scratch between the replays
+        assert g.rt.hipGraphLaunch(run, stream) == 0
+        lib.iris_dev_sync()
+        assert np.array_equal(dev.get(out, (seq, hd), np.uint16), want), f"replay {replay}"
+    g.rt.hipGraphExecDestroy(run)
+    dev.free_all()
