@@ -16,18 +16,29 @@
  * bf16 is the B operand of the second product without leaving the registers.
  * The row sum comes from one more product per tile with an all-ones A operand.
  *
- * Tiles of 32 keys: K and V tile are 32 KB each, two stages of each = 128 KB of
- * LDS, filled by global_load_lds_dwordx4 (a wave has no registers to stage
- * them through): one instruction moves one 1 KB tile row, each wave 8 rows of
- * K and 8 of V per tile, spread over the k-steps of the score product. The
- * loop is skewed by one tile: turn t multiplies the scores of tile t + 1 and
- * the values of tile t, so that K of tile t + 2 and V of tile t + 1 (requested
- * at the start of the turn into the stages the previous turn read last) have a
- * whole turn to arrive; one barrier per turn. Rows are unpadded; the 16 B
- * chunk c of row r sits in slot c ^ 2 (r % 8) of its 256 B group, the
- * permutation applied to the source address of the lane that fills the slot
- * (same conflict-free pattern as the head_dim-128 kernel: a row is a multiple
- * of 256 B there and here).
+ * Tiles of 32 keys: a K or V tile is 32 KB, three K stages and two V stages are
+ * all 160 KB of the LDS, filled by global_load_lds_dwordx4 (a wave has no
+ * registers to stage them through): one instruction moves one 1 KB tile row,
+ * each wave 8 rows of K and 8 of V per tile. The loop is skewed: turn t
+ * multiplies the scores of tile t + 1, then the values of tile t, then takes
+ * the softmax of tile t + 1. V of tile t + 1 is requested during the score
+ * products and K of tile t + 3 during the value products, one row every
+ * eighth product: the CU's one load path runs half busy all the time instead
+ * of saturated for a part of the turn (a request then holds the wave about 20
+ * cycles, not 100), and every request has at least half a turn to land before
+ * the turn's one barrier. Rows are unpadded; the 16 B chunk c of row r sits in
+ * slot c ^ 2 (r % 8) of its 256 B group, the permutation applied to the source
+ * address of the lane that fills the slot (same conflict-free pattern as the
+ * head_dim-128 kernel: a row is a multiple of 256 B there and here).
+ *
+ * What a wave that is alone on its SIMD overlaps with its own products, as
+ * measured here on timing-only variants (16384 tokens, 415 us): memory
+ * instructions, one per gap between two products (operand reads bunched at
+ * the head of a group of four products: +2 %); vector ALU work not at all (the
+ * softmax costs 58 us whether it stands in one block, as it does, or is dealt
+ * out into the gaps between the score products of the next tile). Without
+ * softmax, requests, operand reads and barrier the products alone run at 1.8
+ * PFLOP/s, the power limit of the chip for this instruction.
  *
  * 128 queries per workgroup make few workgroups (16384 tokens: 128 for 256
  * CUs), so the keys of a head may be cut into `splits` ranges, one workgroup
