@@ -622,6 +622,22 @@ def machine_ceilings(dev, hip, stream):
     cp_small = min(event_time(hip, stream, lambda i: mb.iris_mb_copy(stream, *pair(i), small), 48) for _ in range(3))
     rd_small = min(event_time(hip, stream, lambda i: mb.iris_mb_read(stream, _vp(ring[i % 24]), small, sink), 48) for _ in range(3))
     wr_small = min(event_time(hip, stream, lambda i: mb.iris_mb_write(stream, _vp(ring[i % 24]), small), 48) for _ in range(3))
+    # a SIMD's matrix core and its vector ALU, fed by two different waves: each stream alone, then both together
+    mb.iris_mb_mfma_with_valu.argtypes = [_vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int]
+    two = {}
+    for kind, name, per in ((1, "v_fma_f32", 12), (2, "v_exp_f32", 10), (3, "one_exp_per_two_fma", 11)):
+        mi = 6000
+        vi = mi * 8 * 16 // (16 * per)
+        run = lambda m, v: min(event_time(hip, stream, lambda i: mb.iris_mb_mfma_with_valu(stream, sink, 256, m, v, kind), 2) for _ in range(2))
+        run(16, 16)
+        a_ms, v_ms, both_ms = run(mi, 0), run(0, vi), run(mi, vi)
+        two[name] = {"products_alone_us": round(a_ms * 1e3, 1), "vector_alone_us": round(v_ms * 1e3, 1),
+                     "together_us": round(both_ms * 1e3, 1), "together_over_longer": round(both_ms / max(a_ms, v_ms), 3),
+                     "vector_cycles_per_instruction_alone": round(v_ms * 1e-3 * 2.4e9 / (vi * 16), 1)}
+    two["note"] = ("256 blocks of eight waves, two per SIMD: waves 0-3 issue 16x16x32 products on constant operands, waves 4-7 "
+                   "independent vector instructions of one kind. together_over_longer near 1: the two streams run at the same "
+                   "time when they come from different waves; a wave that is alone issues one vector instruction per ~10 "
+                   "cycles (cycles at the nominal 2.4 GHz)")
     dev.check()
     for p in [sink, a, b, ops] + ring:
         lib.iris_dev_free(p)
@@ -634,7 +650,7 @@ def machine_ceilings(dev, hip, stream):
             "write_only_27mib_cold_gbps": round(small / wr_small / 1e6, 1), "write_only_27mib_cold_us": round(wr_small * 1e3, 2),
             "note": "bytes counted read + written for the copies, one direction for the one-way streams; 27 MiB series "
                     "over 24 rotating buffers (648 MiB > the Infinity Cache), back-to-back launches between two events"}
-    return {"streaming_yardsticks": yard,
+    return {"streaming_yardsticks": yard, "matrix_and_vector_from_two_waves": two,
             "inplace_update_27mib_cold_us": round(rw_small * 1e3, 2),
             "inplace_update_27mib_cold_gbps": round(2 * small / rw_small / 1e6, 1),
             "mfma_only_tflops": round(mfma, 1), "mfma_only_frac_of_peak": round(mfma / PEAK_BF16_TFLOPS, 4),

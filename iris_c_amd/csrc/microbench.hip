@@ -163,9 +163,63 @@ __global__ void __launch_bounds__(256) k_exp(float *sink, int iters) {
     if (s == 12345.678f) sink[0] = s;
 }
 
+/* Do a SIMD's matrix core and its vector ALU work at the same time? A block of eight waves, two per SIMD: waves 0-3
+ * issue `mfma_iters` x 8 independent 16x16x32 products, waves 4-7 `valu_iters` x 16 independent vector instructions of
+ * one kind (1: v_fma_f32, 2: v_exp_f32, 3: the softmax's mix, one exponential per two others). Either count may be 0.
+ * Timed three ways by the host (each alone, both together): together = the longer of the two means they overlap,
+ * together = the sum means the SIMD does one or the other. Constant operands, so that the clock does not move. */
+template <int KIND, int ACC>
+__global__ void __launch_bounds__(512) k_mfma_with_valu(float *sink, int mfma_iters, int valu_iters) {
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (wave < 4) {
+        f32x4 acc[8];
+        for (int a = 0; a < 8; a++) acc[a] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        uint4 raw = make_uint4(0x3f803f80u + threadIdx.x, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
+        bf16x8 x = __builtin_bit_cast(bf16x8, raw), y = x;
+        for (int i = 0; i < mfma_iters; i++) {
+#pragma unroll
+            for (int a = 0; a < 8; a++) {
+                if (ACC == 0) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc[a]) : "v"(x), "v"(y));
+                else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[a]) : "v"(x), "v"(y));
+            }
+        }
+        float t = 0.0f;
+        for (int a = 0; a < 8; a++) t += acc[a][0] + acc[a][3];
+        if (t == 12345.678f) sink[0] = t;
+    } else {
+        float v[16];
+        for (int j = 0; j < 16; j++) v[j] = -0.5f - threadIdx.x * 1e-3f - 0.01f * j;
+        const float c = 0.999f, d = -1e-3f;
+        for (int i = 0; i < valu_iters; i++) {
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                if (KIND == 1 || (KIND == 3 && j % 3 != 0)) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v[j]) : "v"(c), "v"(d));
+                else asm volatile("v_exp_f32 %0, %0" : "+v"(v[j]));
+            }
+        }
+        float t = 0.0f;
+        for (int j = 0; j < 16; j++) t += v[j];
+        if (t == 12345.678f) sink[0] = t;
+    }
+}
+
 }  // namespace
 
 extern "C" {
+int iris_mb_mfma_with_valu(void *stream, float *sink, int blocks, int mfma_iters, int valu_iters, int kind) {
+    /* kind: 1 v_fma_f32, 2 v_exp_f32, 3 their mix; + 16: the products' accumulators in AGPRs instead of VGPRs */
+    const dim3 g(blocks), b(512);
+    hipStream_t st = (hipStream_t)stream;
+    switch (kind) {
+    case 1: hipLaunchKernelGGL((k_mfma_with_valu<1, 0>), g, b, 0, st, sink, mfma_iters, valu_iters); break;
+    case 2: hipLaunchKernelGGL((k_mfma_with_valu<2, 0>), g, b, 0, st, sink, mfma_iters, valu_iters); break;
+    case 3: hipLaunchKernelGGL((k_mfma_with_valu<3, 0>), g, b, 0, st, sink, mfma_iters, valu_iters); break;
+    case 17: hipLaunchKernelGGL((k_mfma_with_valu<1, 1>), g, b, 0, st, sink, mfma_iters, valu_iters); break;
+    case 18: hipLaunchKernelGGL((k_mfma_with_valu<2, 1>), g, b, 0, st, sink, mfma_iters, valu_iters); break;
+    default: hipLaunchKernelGGL((k_mfma_with_valu<3, 1>), g, b, 0, st, sink, mfma_iters, valu_iters); break;
+    }
+    return (int)hipGetLastError();
+}
 int iris_mb_mfma(void *stream, float *sink, int blocks, int iters) {
     hipLaunchKernelGGL(k_mfma_peak, dim3(blocks), dim3(256), 0, (hipStream_t)stream, sink, iters);
     return (int)hipGetLastError();
