@@ -95,6 +95,29 @@ def test_vae_16384_tokens_sampled_rows_and_constant_values(dev, orc):
     assert np.array_equal(out2, np.tile(buf[9, 2 * HD:], (seq, 1)))
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", [1, 2])
+def test_random_shapes(dev, orc, seed):
+    """Seeded random sweep at head_dim 512: 32 .. 1500 keys (ragged against the tiles of 32 keys and, through the
+    launcher's choice, against every number of key ranges), 1 .. 700 queries, one to three kv heads with one or two
+    query heads each, padded row strides, two scales and two input spreads."""
+    rng = np.random.default_rng(seed)
+    for case in range(25):
+        kv = int(rng.choice([1, 1, 2, 3]))
+        heads = kv * int(rng.choice([1, 1, 2]))
+        seq_k = int(rng.integers(32, 1500))
+        seq_q = seq_k if rng.random() < 0.5 else int(rng.integers(1, 700))
+        qd, kd = heads * HD, kv * HD
+        ldi = qd + 2 * kd + int(rng.choice([0, 0, 8, 64]))
+        buf = O.f32_to_bf16((rng.standard_normal((max(seq_q, seq_k), ldi)) * rng.choice([0.3, 1.0])).astype(np.float32))
+        scale = float(rng.choice([1 / np.sqrt(HD), 0.02]))
+        what = f"seed {seed} case {case}: q {seq_q} k {seq_k} heads {heads}/{kv} ldi {ldi} scale {scale:.4f} ranges {plan(dev.lib, seq_q, seq_k, heads)[0]}"
+        out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, HD, scale)
+        assert kernel == "fa_hd512", what
+        want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, HD, scale)
+        assert_parity(O.bf16_to_f32(out), want, what)
+
+
 # ------------------------------------------------------------------ every number of key ranges
 def launch_with_ranges(dev, buf, ldi, seq_q, seq_k, heads, kv, scale, splits):
     lib = dev.lib
