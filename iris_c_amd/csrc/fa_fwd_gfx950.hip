@@ -170,6 +170,17 @@ __device__ __forceinline__ const uint16_t *scalar_ptr(const uint16_t *p) {
     return (const uint16_t *)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
 
+/* The same for a pointer that an asm load reads right away. v_readfirstlane is a vector instruction, and a memory
+ * instruction must not read a scalar register within five wait states of a vector instruction writing it; the
+ * compiler places those wait states in front of the memory instructions it issues itself, not in front of an asm
+ * statement. (Unsettled, the load could be issued with the register's previous contents: in practice the old high
+ * half of the address, i.e. wrong only across a 4 GB boundary.) */
+__device__ __forceinline__ const uint16_t *settled_scalar_ptr(const uint16_t *p) {
+    p = scalar_ptr(p);
+    asm volatile("s_nop 4" : "+s"(p));
+    return p;
+}
+
 /* The compiler reserves M0 for its own short-lived uses and remarks on seeing it in a clobber list;
  * naming it is still what tells it that a value it placed there does not survive the statement. */
 #pragma clang diagnostic push
@@ -197,7 +208,7 @@ __device__ __forceinline__ void load_tile(uint16_t *stage, const uint16_t *kt, c
 #pragma unroll
         for (int part = 0; part < NI / 16; part++) {
             const bool is_v = wave * NI + 16 * part >= 16;
-            const uint16_t *src = scalar_ptr(is_v ? vt : kt);
+            const uint16_t *src = settled_scalar_ptr(is_v ? vt : kt);
             uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(stage + (is_v ? K_TILE : 0)));
             const size_t step = 4 * (size_t)ldi;
 #pragma unroll
@@ -811,7 +822,7 @@ k_fa_short_hd128(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict
     auto request_v = [&](int it) {
         const int kn = it * BN;
         if (kn + BN <= seq_k) {
-            const uint16_t *src = scalar_ptr(vbase + (size_t)kn * ldi);
+            const uint16_t *src = settled_scalar_ptr(vbase + (size_t)kn * ldi);
             uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(stage));
             const size_t step = 4 * (size_t)ldi;
 #pragma unroll

@@ -1,12 +1,10 @@
 """The head_dim-512 attention kernel (one wave per SIMD owns 32 whole queries; the VAE mid-block call of the
 reference, iris_vae.c:1112-1124) through the C ABI and, for the number of key ranges, through the kernel's own
 launcher, against the fp32 CPU oracle on identical bf16 inputs. Bars as in test_gpu_attention.py.
-The planner and the instruction-level check at the end need no GPU.
+The planner test at the end needs no GPU.
 """
 import ctypes as C
 import os
-import re
-import subprocess
 
 import numpy as np
 import pytest
@@ -181,41 +179,3 @@ def test_planner_never_leaves_a_range_empty():
         assert need == (0 if splits == 1 else seq_q * heads * splits * (HD + 2) * 4)
     assert plan(lib, 16384, 16384, 1)[0] == 2                 # 128 workgroups of 128 queries on 256 CUs
     assert plan(lib, 128, 64, 1)[0] == 1
-
-
-def test_no_ordinary_instruction_feeds_an_asm_matrix_instruction_directly():
-    """The kernel's matrix instructions are asm statements, and the compiler places the wait states that a matrix
-    instruction needs behind an ordinary vector instruction writing one of its operands only for matrix
-    instructions it issues itself. (A v_mov materialising the all-ones operand right in front of the row-sum
-    product made a quarter of the lanes read the old register contents.) So the generated code is scanned: no vector
-    ALU instruction may write a register that an asm matrix instruction reads within the next three instructions."""
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    if not os.path.exists(hipcc):
-        pytest.skip("no hipcc here")
-    src = os.path.join(ROOT, "iris_c_amd", "csrc", "fa_fwd_hd512_gfx950.hip")
-    r = subprocess.run([hipcc, "-O3", "--offload-arch=gfx950", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-                        "-packed-fp32-ops", "-I" + os.path.join(ROOT, "iris_c_amd", "csrc"), "-I" + os.path.join(ROOT, "include"),
-                        "--cuda-device-only", "-S", "-o", "-", src], capture_output=True, text=True)
-    assert r.returncode == 0, r.stderr[-2000:]
-    ins = [l.strip() for l in r.stdout.splitlines()]
-    ins = [l for l in ins if l and not l.startswith((";", ".")) and not l.endswith(":")]
-
-    def regs(tok):
-        m = re.match(r"([va])\[(\d+):(\d+)\]", tok)
-        if m:
-            return {(m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1)}
-        m = re.match(r"([va])(\d+)$", tok)
-        return {(m.group(1), int(m.group(2)))} if m else set()
-
-    products = 0
-    for i, l in enumerate(ins):
-        if not l.startswith("v_mfma"):
-            continue
-        products += 1
-        src_regs = set().union(*[regs(t.strip()) for t in l.split(None, 1)[1].split(",")[1:]])
-        for back in (1, 2, 3):
-            p = ins[i - back]
-            if p.startswith("v_") and not p.startswith("v_mfma"):
-                dst = regs(p.split(None, 1)[1].split(",")[0].strip())
-                assert not (dst & src_regs), f"{p}  feeds  {l}"
-    assert products > 300                                     # both instantiations were scanned
