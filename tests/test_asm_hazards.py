@@ -9,8 +9,11 @@ own business and are checked here on the code of every build:
   instructions (a v_mov materialising the all-ones operand of the row-sum product right in front of it made a quarter
   of the lanes read the old register contents);
 * a vector instruction that writes a scalar register (v_readfirstlane, v_readlane, v_cmp) must be five wait states
-  ahead of a memory instruction that reads that register (an unsettled pointer is read with its old high half).
+  ahead of a memory instruction that reads that register (an unsettled pointer is read with its old high half);
+* the data registers of a store of more than 8 bytes must not be written by a vector instruction within the two wait
+  states behind the store (the norm+rope kernel's streaming stores are asm statements).
 """
+import functools
 import os
 import re
 import subprocess
@@ -22,6 +25,7 @@ CSRC = os.path.join(ROOT, "iris_c_amd", "csrc")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
+@functools.lru_cache(maxsize=None)
 def isa(name):
     if not os.path.exists(HIPCC):
         pytest.skip("no hipcc here")
@@ -90,3 +94,18 @@ def test_scalar_registers_written_by_vector_instructions_settle_before_memory_in
             m = re.match(r"s_nop (\d+)", p)
             waits += int(m.group(1)) + 1 if m else 1
     assert loads > 0
+
+
+@pytest.mark.parametrize("name", sorted(f for f in os.listdir(CSRC) if f.endswith(".hip")))
+def test_data_registers_of_a_wide_store_are_left_alone_right_behind_it(name):
+    ins = isa(name)
+    for i, l in enumerate(ins):
+        if not re.match(r"(global|flat|scratch)_store_dwordx[34]", l):
+            continue
+        data = vregs(operands(l)[1])
+        waits = 0
+        for p in ins[i + 1:i + 3]:
+            if waits < 2 and p.startswith("v_"):
+                assert not (vregs(operands(p)[0]) & data), f"{name}: {p}  overwrites the data of  {l}"
+            m = re.match(r"s_nop (\d+)", p)
+            waits += int(m.group(1)) + 1 if m else 1
