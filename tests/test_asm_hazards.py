@@ -10,6 +10,8 @@ own business and are checked here on the code of every build:
   of the lanes read the old register contents);
 * a vector instruction that writes a scalar register (v_readfirstlane, v_readlane, v_cmp) must be five wait states
   ahead of a memory instruction that reads that register (an unsettled pointer is read with its old high half);
+* the result registers of an asm matrix instruction must not be read or written by any other kind of instruction
+  within eleven wait states of it (the product has to leave the matrix core first);
 * the data registers of a store of more than 8 bytes must not be written by a vector instruction within the two wait
   states behind the store (the norm+rope kernel's streaming stores are asm statements).
 """
@@ -107,5 +109,23 @@ def test_data_registers_of_a_wide_store_are_left_alone_right_behind_it(name):
         for p in ins[i + 1:i + 3]:
             if waits < 2 and p.startswith("v_"):
                 assert not (vregs(operands(p)[0]) & data), f"{name}: {p}  overwrites the data of  {l}"
+            m = re.match(r"s_nop (\d+)", p)
+            waits += int(m.group(1)) + 1 if m else 1
+
+
+@pytest.mark.parametrize("name", ["fa_fwd_hd512_gfx950.hip", "gemm_conv_gfx950.hip"])
+def test_results_of_asm_matrix_instructions_are_left_alone_until_they_have_left_the_matrix_core(name):
+    ins = isa(name)
+    for i, l in enumerate(ins):
+        if not l.startswith("v_mfma"):
+            continue
+        result = vregs(operands(l)[0])
+        waits = 0
+        for p in ins[i + 1:i + 14]:
+            if waits >= 11:
+                break
+            if not p.startswith(("v_mfma", "s_")):
+                touched = set().union(*[vregs(t) for t in operands(p)]) if operands(p) else set()
+                assert not (touched & result), f"{name}: {p}  touches the result of  {l}  {waits} wait states behind it"
             m = re.match(r"s_nop (\d+)", p)
             waits += int(m.group(1)) + 1 if m else 1
