@@ -1,8 +1,9 @@
 /*
- * Flash-attention forward for gfx950, head_dim 512, no mask, not causal: the
- * VAE mid-block attention of the reference (one head of 512 over every latent
- * position, iris_vae.c:1112-1124; operator contract iris_dev.h:83-92). bf16
- * in, f32 accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16).
+ * Flash-attention forward for gfx950, head_dim 512: the VAE mid-block
+ * attention of the reference (one head of 512 over every latent position,
+ * iris_vae.c:1112-1124; operator contract iris_dev.h:83-92, whose key mask
+ * and causal limit are template options here). bf16 in, f32 accumulation on
+ * the matrix cores (v_mfma_f32_16x16x32_bf16).
  *
  * One wave per SIMD, each with the whole register file: a wave owns 32 queries
  * and all 512 output dims of them, O^T as 64 accumulator blocks of 16 dims x 16
@@ -44,6 +45,11 @@
  * CUs), so the keys of a head may be cut into `splits` ranges, one workgroup
  * per (query tile, range); these write their unnormalised O (f32), running max
  * and row sum to a scratch buffer and k_fa_hd512_merge combines them.
+ *
+ * A key mask arrives as one word per key tile (k_pack_key_mask, a launch in
+ * front); the walk over the keys ends at the last tile that has a valid key.
+ * A causal call walks the tiles in front of each workgroup's last query; its
+ * workgroups differ in length and are numbered by falling length.
  */
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -112,18 +118,61 @@ struct Partials {
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
 
-template <bool SPLIT>
+/* The workgroups of a causal call in the order of falling length. With `step` = tiles_per_split / 4 query tiles per key
+ * range, the pair (query tile qt, range r) walks min(4 (qt + 1) - r * tiles_per_split, tiles_per_split) tiles, which
+ * depends on qt - r * step only; pairs with qt - r * step < 0 have none and get no number. Number j -> how far the
+ * pair's qt - r * step lies behind the last query tile, and r: at distance u the ranges 0 .. min(u / step, splits - 1)
+ * exist. */
+__host__ __device__ inline void causal_pair(int j, int step, int splits, int &behind, int &r) {
+    if (step == 0) { behind = j / splits; r = j % splits; return; }
+    int k = 0, first = 0;                            /* first: the number of the first pair with u / step == k */
+    while (k < splits - 1 && j >= first + step * (k + 1)) { first += step * (k + 1); k++; }
+    behind = k * step + (j - first) / (k + 1);
+    r = (j - first) % (k + 1);
+}
+__host__ inline int causal_pairs(int q_tiles, int step, int splits) {
+    if (step == 0) return q_tiles * splits;
+    int n = 0;
+    for (int u = 0; u < q_tiles; u++) n += u / step + 1 < splits ? u / step + 1 : splits;
+    return n;
+}
+
+/* SPLIT: one of several key ranges (partial results to `part`). CAUSAL: query i ignores keys j > i; a workgroup walks
+ * the tiles of its range up to its last query, and the workgroups are numbered by falling length. MASK:
+ * `mask_words[t]` holds the valid keys of key tile t as k_pack_key_mask left them. */
+template <bool SPLIT, bool CAUSAL, bool MASK>
 __global__ void __launch_bounds__(THREADS, 1)
 k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ q,
                const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
                int seq_q, int seq_k, int heads, int q_tiles, int splits, int tiles_per_split,
-               int total_work, int work_per_xcd, int kv_group, float scale_log2, Partials part) {
-    extern __shared__ __align__(16) uint16_t lds[];     /* K stage 0, 1 | V stage 0, 1 */
+               int total_work, int work_per_xcd, int kv_group, float scale_log2, Partials part,
+               const uint32_t *__restrict__ mask_words) {
+    extern __shared__ __align__(16) uint16_t lds[];     /* K stages 0, 1, 2 | V stages 0, 1 */
 
-    const int work = (blockIdx.x % XCDS) * work_per_xcd + blockIdx.x / XCDS;
-    if (work >= total_work) return;
-    const int qt = work % q_tiles, rest = work / q_tiles;
-    const int split = rest % splits, head = rest / splits;
+    int qt, split, head;
+    if (CAUSAL) {
+        /* Workgroups differ in length: query tile qt has 4 (qt + 1) key tiles in front of it, of which range r holds
+         * those from r * tiles_per_split on. The hardware deals workgroup b to XCD b % 8 and every XCD starts its own
+         * in order, so they are numbered by falling length (causal_pair), heads innermost: neighbours are equally
+         * long, which also gives every XCD the same mix. Only pairs that have a key tile get a number. An XCD has been
+         * seen to hand its workgroups to its four shader engines in turn and to wait with the next one until the
+         * engine whose turn it is has a free CU, so every other group of 32 (8 XCDs x 4 engines) runs backwards: the
+         * engine that got the shortest of one group, and is free first, gets the longest of the next. (256 CUs hold
+         * eight groups at a time, so it is an odd group that meets an even one there.) */
+        const int slot = (blockIdx.x & 32) ? (blockIdx.x & ~31) | (31 - (blockIdx.x & 31)) : blockIdx.x;
+        if (slot >= total_work) return;
+        int behind;
+        causal_pair(slot / heads, tiles_per_split / 4, splits, behind, split);
+        head = slot % heads;
+        qt = q_tiles - 1 - behind + split * (tiles_per_split / 4);
+    } else {
+        const int work = (blockIdx.x % XCDS) * work_per_xcd + blockIdx.x / XCDS;
+        if (work >= total_work) return;
+        const int rest = work / q_tiles;
+        qt = work % q_tiles;
+        split = rest % splits;
+        head = rest / splits;
+    }
     const int kvh = head / kv_group;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -132,8 +181,40 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 
     const uint16_t *kbase = scalar_ptr(k + (size_t)kvh * HD);
     const uint16_t *vbase = scalar_ptr(v + (size_t)kvh * HD);
-    const int t_begin = split * tiles_per_split;
-    const int nt = min((seq_k + BN - 1) / BN - t_begin, tiles_per_split);      /* >= 1: the launcher makes no empty range */
+    int t_begin = split * tiles_per_split;
+    /* tiles of this workgroup's range: >= 1 when not causal (the launcher makes no empty range) */
+    const int k_end = CAUSAL ? min(seq_k, qt * BM + BM) : seq_k;
+    int nt = min((k_end + BN - 1) / BN - t_begin, tiles_per_split);
+    if (SPLIT && CAUSAL && nt <= 0) return;          /* the range begins behind the last query: the merge skips it too */
+    if (MASK) {
+        /* A padding mask: the walk ends with the last tile of the sequence that has a valid key. Every workgroup finds
+         * it by itself (at most seven words per thread); a call that is not causal then cuts the tiles up to there
+         * into its ranges instead of all tiles, so that the ranges stay equally long. */
+        int last = 0;
+        for (int i = threadIdx.x; i < (seq_k + BN - 1) / BN; i += THREADS)
+            if (mask_words[i]) last = i;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) last = max(last, __shfl_xor(last, off));
+        int *share = reinterpret_cast<int *>(lds);
+        if ((threadIdx.x & 63) == 0) share[threadIdx.x >> 6] = last;
+        lds_barrier();
+        last = max(max(share[0], share[1]), max(share[2], share[3]));
+        lds_barrier();                               /* before the first tile lands on these words */
+        last = __builtin_amdgcn_readfirstlane(last);
+        if (CAUSAL) {
+            nt = min(nt, last + 1 - t_begin);
+        } else {
+            const int per = (last + splits) / splits;
+            t_begin = split * per;
+            nt = min(last + 1 - t_begin, per);
+        }
+        if (SPLIT && nt <= 0) {                      /* nothing valid in this range: (max, sum) = (-inf, 0), which the merge skips */
+            const int row = qt * BM + threadIdx.x;
+            if (threadIdx.x < BM && row < seq_q)
+                *reinterpret_cast<f32x2 *>(part.ml + 2 * (((size_t)split * heads + head) * seq_q + row)) = f32x2{-INFINITY, 0.0f};
+            return;
+        }
+    }
 
     /* LDS: K stages 0, 1, 2 | V stages 0, 1 (TILE elements each). Read offsets in elements from the start of the LDS.
      * K operand (key block mb, k-step ks): row 16 mb + li, chunk 4 ks + lg = 16 (ks / 4) + (4 (ks % 4) + lg); the
@@ -263,10 +344,15 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
      * score of the wave exceeds it by more than 2^8; that test needs no cross-lane traffic (the four lanes of a
      * query share the bound). ---- */
     u32x4 pw[2];
-    auto softmax = [&](int tile) INLINE {
+    auto softmax = [&](int tile, uint32_t mask_word) INLINE {
         const int k0 = (t_begin + tile) * BN;
-        if (k0 + BN > seq_k) {                       /* the last tile of the sequence: moved back by k0 + 32 - seq_k keys, which are masked */
-            const unsigned mine = (~0u << (k0 + BN - seq_k)) >> (4 * lg);
+        /* valid keys of the tile as a wave-uniform set: the last tile of the sequence is moved back by k0 + 32 - seq_k
+         * keys, which belong to the tile before; with a key mask the packed word says all of this already */
+        uint32_t valid = ~0u;
+        if (k0 + BN > seq_k) valid = ~0u << (k0 + BN - seq_k);
+        if (MASK) valid = mask_word;
+        if (valid != ~0u) {
+            const unsigned mine = valid >> (4 * lg);
 #pragma unroll
             for (int mb = 0; mb < 2; mb++)
 #pragma unroll
@@ -275,6 +361,19 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 #pragma unroll
                         for (int nb = 0; nb < 2; nb++) s[mb][nb][r] = -INFINITY;
                     }
+        }
+        if (CAUSAL) {
+            const int first = min(k0, seq_k - BN);              /* the key in row 0 of the tile as it was loaded */
+            if (first + BN - 1 > wq0) {                          /* wave-uniform: some key lies behind the wave's first query */
+                const int lim0 = qrow0 - first - 4 * lg;         /* key offset 16 mb + r is valid iff <= lim0 (+ 16 nb) */
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+#pragma unroll
+                        for (int nb = 0; nb < 2; nb++)
+                            if (16 * mb + r > lim0 + 16 * nb) s[mb][nb][r] = -INFINITY;
+            }
         }
         float lane_max[2];
         bool raise = false;
@@ -365,7 +464,18 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
      * and the softmax that reads its scores; here idle cycles do. */
     scores([](int) INLINE {});
     asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]));
-    softmax(0);
+    /* The words of the key mask are read through the scalar cache two turns at a time and waited for on the spot (the
+     * empty asm consumes them): a scalar load left pending would turn every wait for an LDS operand into a wait for
+     * everything. */
+    auto mask_word = [&](int tile) INLINE {
+        uint32_t w = 0;
+        if (MASK) {
+            w = mask_words[t_begin + min(tile, nt - 1)];
+            asm volatile("" : "+s"(w));
+        }
+        return w;
+    };
+    softmax(0, mask_word(0));
     lds_barrier();                                   /* K stage 0 has no readers any more */
     int kstage = 1;                                  /* where the K operand offsets point: the stage of tile t + 1 */
 #pragma unroll
@@ -378,7 +488,7 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
      * product, so that the four waves keep the CU's one load path half busy all the time instead of saturating it
      * for a part of the turn. At the end of the turn everything but the eight newest requests (K of tile t + 3) must
      * have landed. */
-    auto turn = [&](int t, int par) INLINE {
+    auto turn = [&](int t, int par, uint32_t next_mask_word) INLINE {
         const uint16_t *vrows = tile_rows(vbase, t + 1), *krows = tile_rows(kbase, t + 3);
         scores([&](int i) INLINE {
             if ((i & 7) == 5) request_row(vrows, 3 + (par ^ 1), i >> 3);
@@ -387,7 +497,7 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         values(par, [&](int i) INLINE {
             if ((i & 7) == 5) request_row(krows, kreq, i >> 3);
         });
-        if (t + 1 < nt) softmax(t + 1);
+        if (t + 1 < nt) softmax(t + 1, next_mask_word);
         const int step = kstage == 2 ? -2 * TILE : TILE;
         kstage = kstage == 2 ? 0 : kstage + 1;
 #pragma unroll
@@ -396,8 +506,9 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         lds_barrier();
     };
     for (int t = 0; t < nt; t += 2) {
-        turn(t, 0);
-        if (t + 1 < nt) turn(t + 1, 1);
+        const uint32_t w1 = mask_word(t + 1), w2 = mask_word(t + 2);
+        turn(t, 0, w1);
+        if (t + 1 < nt) turn(t + 1, 1, w2);
     }
     wait_vmcnt<0>();                                  /* nothing may still be on its way into the LDS when it is given back */
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");      /* the last products have left the matrix core */
@@ -436,20 +547,42 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 
 #pragma clang diagnostic pop
 
+/* The key mask as one 32-bit word per key tile, bit j = key j of the tile AS THE KERNEL LOADS IT is valid: the last
+ * tile of a sequence whose length is not a multiple of 32 is moved back to end with it, and the keys it shares with
+ * the tile before count as invalid there. 64 threads = two tiles per block; `words` has room for an even count. */
+__global__ void __launch_bounds__(64)
+k_pack_key_mask(uint32_t *__restrict__ words, const int *__restrict__ key_mask, int seq_k, int tiles) {
+    const int tile = 2 * blockIdx.x + (threadIdx.x >> 5), j = threadIdx.x & 31;
+    const int first = min(tile * BN, seq_k - BN), key = first + j;
+    const bool ok = tile < tiles && key >= tile * BN && key_mask[key] != 0;
+    const unsigned long long both = __ballot(ok);
+    if (threadIdx.x == 0) {
+        words[2 * blockIdx.x] = (uint32_t)both;
+        words[2 * blockIdx.x + 1] = (uint32_t)(both >> 32);
+    }
+}
+
 /* Combines the key ranges of a query: out = sum_r 2^(m_r - m) o_r / sum_r 2^(m_r - m) l_r with m the largest of the
  * maxima. 64 threads per query row, 8 dims each. */
 __global__ void __launch_bounds__(256)
-k_fa_hd512_merge(uint16_t *__restrict__ out, int ldo, Partials part, int seq_q, int heads, int splits) {
+k_fa_hd512_merge(uint16_t *__restrict__ out, int ldo, Partials part, int seq_q, int heads, int splits, int causal_keys,
+                 int tiles_per_split) {
     const size_t rows = (size_t)heads * seq_q;
     const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);       /* head * seq_q + query */
     if (row >= rows) return;
     const int t = threadIdx.x & 63;
+    const size_t head = row / seq_q, qrow = row - head * seq_q;
+    if (causal_keys) {                                /* a causal call of causal_keys keys: ranges behind the query's workgroup were never written */
+        const int keys = min(causal_keys, ((int)qrow / BM + 1) * BM);
+        splits = min(splits, ((keys + BN - 1) / BN + tiles_per_split - 1) / tiles_per_split);
+    }
     float m = -INFINITY;
     for (int r = 0; r < splits; r++) m = fmaxf(m, part.ml[2 * (r * rows + row)]);
     float l = 0.0f, acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     for (int r = 0; r < splits; r++) {
         const f32x2 ml = *reinterpret_cast<const f32x2 *>(part.ml + 2 * (r * rows + row));
-        const float w = ml[0] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ml[0] - m);
+        if (ml[0] == -INFINITY) continue;             /* no valid key in this range */
+        const float w = __builtin_amdgcn_exp2f(ml[0] - m);
         l += w * ml[1];
         const float *po = part.o + (r * rows + row) * HD + 8 * t;
         const f32x4 a = *reinterpret_cast<const f32x4 *>(po), b = *reinterpret_cast<const f32x4 *>(po + 4);
@@ -457,7 +590,6 @@ k_fa_hd512_merge(uint16_t *__restrict__ out, int ldo, Partials part, int seq_q, 
         for (int i = 0; i < 4; i++) { acc[i] += w * a[i]; acc[4 + i] += w * b[i]; }
     }
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    const size_t head = row / seq_q, qrow = row - head * seq_q;
     uint16_t *op = out + qrow * ldo + head * HD + 8 * t;                  /* output rows are 8-byte aligned, not more */
     *reinterpret_cast<uint2 *>(op) = make_uint2(pack_bf16(acc[0] * inv, acc[1] * inv), pack_bf16(acc[2] * inv, acc[3] * inv));
     *reinterpret_cast<uint2 *>(op + 4) = make_uint2(pack_bf16(acc[4] * inv, acc[5] * inv), pack_bf16(acc[6] * inv, acc[7] * inv));
@@ -480,70 +612,127 @@ int cu_count() {
 
 }  // namespace
 
-/* How many key ranges a call is cut into, and the scratch it then needs (0 for one range). Host arithmetic only.
+/* How many key ranges a call is cut into, and the scratch it then needs (partial rows for more than one range, the
+ * packed key mask for a masked call; 0 for neither). Host arithmetic only.
  * Fitted to every number of ranges at 256 .. 50176 tokens: a turn of 32 keys takes a workgroup 1.6 us when all CUs
  * are busy and 1.3 us when few are (the clock follows the load), a round of workgroups costs its turns plus about
  * 8 us of start and end, and the merge reads and writes the partial rows at about 6 TB/s (they are still in the
  * caches) behind a launch of 4 us and half a microsecond per range. The choice is within 3 % of the best count from
- * 9216 tokens on and within 6 % below (where every count from 4 to 8 is within 10 % of every other). */
-extern "C" size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int *splits_out) {
+ * 9216 tokens on and within 6 % below (where every count from 4 to 8 is within 10 % of every other).
+ * A causal call has workgroups of 4, 8, 12, ... tiles: it takes the longer of its longest workgroup and of all its
+ * turns spread over the CUs, and ranges shorten the former; ranges that begin behind a workgroup's last query do
+ * not exist, in the kernel and in the merge. Fitted to 1 .. 8 ranges at 1024 .. 30000 tokens: the choice costs 1 %
+ * on average against the best count. */
+extern "C" size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int causal, int masked, int *splits_out) {
     const long cus = cu_count();
-    const long tiles = (seq_k + BN - 1) / BN, wgs = (long)((seq_q + BM - 1) / BM) * heads;
+    const long tiles = (seq_k + BN - 1) / BN, q_tiles = (seq_q + BM - 1) / BM, wgs = q_tiles * heads;
     const double rows_mb = (double)seq_q * heads * HD * 4 / 1e6;          /* one range's partial O, MB */
     double best = 0.0;
     int best_s = 1;
     for (int s = 1; s <= 8 && s <= tiles; s++) {
         const long per = (tiles + s - 1) / s, ranges = (tiles + per - 1) / per;
         if (ranges != s) continue;
-        const long full = wgs * ranges / cus, rest = wgs * ranges % cus;
-        double us = full * (per * 1.6 + 8.0);
-        if (rest) us += per * (1.3 + 0.3 * (double)rest / cus) + 8.0;
-        if (ranges > 1) us += 4.0 + 0.5 * ranges + 2.0 * ranges * rows_mb / 6.0;          /* MB / (TB/s) = us */
+        double us;
+        if (causal) {
+            long turns = 0, filled = 0;              /* over the query tiles of a head: tiles walked, ranges that are not empty */
+            for (long qt = 0; qt < q_tiles; qt++) {
+                const long keys = qt * BM + BM < seq_k ? qt * BM + BM : seq_k, mine = (keys + BN - 1) / BN;
+                turns += mine;
+                filled += (mine + per - 1) / per;
+            }
+            /* in turns: the longest workgroup when all run at once, else all turns spread over the CUs plus a ragged
+             * end; a turn costs 1.2 us on an empty machine and 1.7 us on a full one */
+            const double longest = (double)(per < tiles ? per : tiles), spread = (double)turns * heads / cus + 0.2 * longest;
+            const double span = filled * heads <= cus || longest > spread ? longest : spread;
+            us = span * (1.2 + 0.5 * (double)turns * heads / (cus * span)) + 10.0 * (double)((filled * heads + cus - 1) / cus);
+            if (ranges > 1) us += 4.0 + 0.5 * ranges + 2.0 * (double)filled * heads * (BM * HD * 4 / 1e6) / 6.0;
+        } else {
+            const long full = wgs * ranges / cus, rest = wgs * ranges % cus;
+            us = full * (per * 1.6 + 8.0);
+            if (rest) us += per * (1.3 + 0.3 * (double)rest / cus) + 8.0;
+            if (ranges > 1) us += 4.0 + 0.5 * ranges + 2.0 * ranges * rows_mb / 6.0;          /* MB / (TB/s) = us */
+        }
         if (s == 1 || us < best * 0.97) { best = us; best_s = s; }
     }
     *splits_out = best_s;
-    if (best_s == 1) return 0;
-    const size_t rows = (size_t)seq_q * heads * best_s;
-    return rows * HD * sizeof(float) + rows * 2 * sizeof(float);
+    const size_t rows = best_s == 1 ? 0 : (size_t)seq_q * heads * best_s;
+    const size_t words = masked ? ((size_t)tiles + 2) / 2 * 2 : 0;
+    return rows * HD * sizeof(float) + rows * 2 * sizeof(float) + words * sizeof(uint32_t);
 }
 
-/* head_dim 512, no mask, not causal; rows 16-byte aligned (ldi % 8 == 0, ldo % 4 == 0), seq_k >= 32, scale > 0.
- * `splits` and `scratch` as iris_hip_fa_hd512_plan says for the same sizes (scratch may be null for one range). */
-extern "C" int iris_hip_fa_hd512(void *stream, uint16_t *out, int ldo, const uint16_t *q,
-                                 const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
-                                 int seq_k, int heads, int kv_heads, float scale, int splits, void *scratch) {
-    hipStream_t st = (hipStream_t)stream;
-    const int tiles = (seq_k + BN - 1) / BN;
-    if (seq_k < BN || splits < 1 || splits > tiles || (splits > 1 && !scratch)) return (int)hipErrorInvalidValue;
-    const int per = (tiles + splits - 1) / splits;
-    if ((tiles + per - 1) / per != splits) return (int)hipErrorInvalidValue;      /* an empty range */
+/* The numbering of a causal call's workgroups, for inspection on the host: pair `number` of a call with q_tiles query
+ * tiles and ranges of tiles_per_split key tiles -> its query tile and range; returns how many pairs there are. */
+extern "C" int iris_hip_fa_hd512_causal_order(int number, int q_tiles, int tiles_per_split, int splits, int *qt, int *range) {
+    const int pairs = causal_pairs(q_tiles, tiles_per_split / 4, splits);
+    if (number >= 0 && number < pairs) {
+        int behind;
+        causal_pair(number, tiles_per_split / 4, splits, behind, *range);
+        *qt = q_tiles - 1 - behind + *range * (tiles_per_split / 4);
+    }
+    return pairs;
+}
+
+namespace {
+template <bool SPLIT, bool CAUSAL, bool MASK>
+int launch_hd512(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi,
+                 int seq_q, int seq_k, int heads, int kv_heads, float scale, int splits, int per, Partials part,
+                 const uint32_t *mask_words) {
     static bool configured = false;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd512<false>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd512<SPLIT, CAUSAL, MASK>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd512<true>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
         if (e != hipSuccess) return (int)e;
         configured = true;
     }
     const int q_tiles = (seq_q + BM - 1) / BM;
-    const int total = q_tiles * heads * splits;
-    const int per_xcd = (total + XCDS - 1) / XCDS;
-    const size_t rows = (size_t)seq_q * heads * splits;
+    const int total = (CAUSAL ? causal_pairs(q_tiles, per / 4, splits) : q_tiles * splits) * heads;
+    const int per_xcd = CAUSAL ? (total + 31) / 32 * 4 : (total + XCDS - 1) / XCDS;     /* causal: whole groups of 32 */
+    hipLaunchKernelGGL((k_fa_fwd_hd512<SPLIT, CAUSAL, MASK>), dim3(per_xcd * XCDS), dim3(THREADS), LDS_BYTES, st, out, ldo, q, k, v,
+                       ldi, seq_q, seq_k, heads, q_tiles, splits, per, total, per_xcd, heads / kv_heads,
+                       scale * 1.4426950408889634f, part, mask_words);
+    return (int)hipGetLastError();
+}
+}  // namespace
+
+/* head_dim 512; rows 16-byte aligned (ldi % 8 == 0, ldo % 4 == 0), seq_k >= 32, scale > 0; key_mask: device int
+ * [seq_k] or null. `splits` and `scratch` (16-byte aligned) as iris_hip_fa_hd512_plan says for the same sizes and
+ * flags; scratch may be null when it says 0 bytes. */
+extern "C" int iris_hip_fa_hd512(void *stream, uint16_t *out, int ldo, const uint16_t *q,
+                                 const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
+                                 int seq_k, int heads, int kv_heads, float scale, int causal, const int *key_mask,
+                                 int splits, void *scratch) {
+    hipStream_t st = (hipStream_t)stream;
+    const int tiles = (seq_k + BN - 1) / BN;
+    if (seq_k < BN || splits < 1 || splits > tiles || ((splits > 1 || key_mask) && !scratch))
+        return (int)hipErrorInvalidValue;
+    const int per = (tiles + splits - 1) / splits;
+    if ((tiles + per - 1) / per != splits) return (int)hipErrorInvalidValue;      /* an empty range */
+    const size_t rows = splits == 1 ? 0 : (size_t)seq_q * heads * splits;
     Partials part = {reinterpret_cast<float *>(scratch), reinterpret_cast<float *>(scratch) + rows * HD};
-    const float scale_log2 = scale * 1.4426950408889634f;
-    if (splits == 1) {
-        hipLaunchKernelGGL((k_fa_fwd_hd512<false>), dim3(per_xcd * XCDS), dim3(THREADS), LDS_BYTES, st, out, ldo, q, k, v,
-                           ldi, seq_q, seq_k, heads, q_tiles, 1, per, total, per_xcd, heads / kv_heads, scale_log2, part);
-        return (int)hipGetLastError();
+    uint32_t *words = nullptr;
+    if (key_mask) {
+        words = reinterpret_cast<uint32_t *>(reinterpret_cast<float *>(scratch) + rows * (HD + 2));
+        hipLaunchKernelGGL(k_pack_key_mask, dim3((unsigned)((tiles + 1) / 2)), dim3(64), 0, st, words, key_mask, seq_k, tiles);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL((k_fa_fwd_hd512<true>), dim3(per_xcd * XCDS), dim3(THREADS), LDS_BYTES, st, out, ldo, q, k, v,
-                       ldi, seq_q, seq_k, heads, q_tiles, splits, per, total, per_xcd, heads / kv_heads, scale_log2, part);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return (int)e;
+    int e;
+    if (causal && splits == 1) {
+        e = key_mask ? launch_hd512<false, true, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, 1, per, part, words)
+                     : launch_hd512<false, true, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, 1, per, part, words);
+    } else if (causal) {
+        e = key_mask ? launch_hd512<true, true, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, splits, per, part, words)
+                     : launch_hd512<true, true, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, splits, per, part, words);
+    } else if (splits == 1) {
+        e = key_mask ? launch_hd512<false, false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, 1, per, part, words)
+                     : launch_hd512<false, false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, 1, per, part, words);
+    } else {
+        e = key_mask ? launch_hd512<true, false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, splits, per, part, words)
+                     : launch_hd512<true, false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, splits, per, part, words);
+    }
+    if (e || splits == 1) return e;
     const size_t merge_rows = (size_t)seq_q * heads;
     hipLaunchKernelGGL(k_fa_hd512_merge, dim3((unsigned)((merge_rows + 3) / 4)), dim3(256), 0, st, out, ldo, part, seq_q,
-                       heads, splits);
+                       heads, splits, causal ? seq_k : 0, per);
     return (int)hipGetLastError();
 }

@@ -70,15 +70,18 @@ int iris_hip_fa_sliced(void *stream, uint16_t *out, int ldo, const uint16_t *q,
                        int heads, int kv_heads, int head_dim, float scale, int causal,
                        const int *key_mask);
 
-/* head_dim 512 without mask or causal limit (the VAE's call): one wave per SIMD owns 32 queries and all 512 output
- * dims; the keys may be cut into ranges that a second launch merges. iris_hip_fa_hd512_plan says how many ranges a
- * call of these sizes takes and returns the bytes of scratch it then needs (0 for one range; host arithmetic, no
- * GPU needed); iris_hip_fa_hd512 wants exactly that `splits` and a scratch of that size, 16-byte aligned, and at
- * least 32 keys. Same argument conditions as iris_hip_fa_hd128 otherwise. */
-size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int *splits);
+/* head_dim 512 and at least 32 keys (the VAE's call; key mask and causal limit as options): one wave per SIMD owns
+ * 32 queries and all 512 output dims; the keys may be cut into ranges that a second launch merges (a causal call
+ * never is). iris_hip_fa_hd512_plan says how many ranges a call of these sizes takes and returns the bytes of scratch
+ * it then needs: partial rows of the ranges, and the packed key mask of a masked call (0 for one range without mask;
+ * host arithmetic, no GPU needed). iris_hip_fa_hd512 wants exactly that `splits` and a scratch of that size, 16-byte
+ * aligned. Same argument conditions as iris_hip_fa_hd128 otherwise. */
+size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int causal, int masked, int *splits);
+/* host arithmetic: workgroup `number` of a causal call -> (query tile, key range); returns the count of workgroups */
+int iris_hip_fa_hd512_causal_order(int number, int q_tiles, int tiles_per_split, int splits, int *qt, int *range);
 int iris_hip_fa_hd512(void *stream, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
                       const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads,
-                      float scale, int splits, void *scratch);
+                      float scale, int causal, const int *key_mask, int splits, void *scratch);
 
 /* Any head_dim (up to IRIS_ATTENTION_Q_IN_LDS_MAX_HEAD_DIM the 8 queries of a workgroup are kept in LDS as f32,
  * beyond it they are read from global memory), any stride / alignment / scale; the rows of q may have a stride

@@ -306,19 +306,21 @@ void iris_dev_head_norm_rope_qk_streams(uint16_t *xq, uint16_t *xk, int ld,
                       split_half);
 }
 
-/* head_dim 256 / 512 on the matrix cores (rows 16-byte aligned). 512 without mask or causal limit, the VAE's call,
- * takes the kernel in which a wave owns 32 whole queries; its key ranges, if it cuts any, leave their partial results
- * in private scratch. Everything else takes the kernel that slices the head dim over the waves. Returns 0 or a HIP
- * error; -1 when the scratch could not be had (already reported). */
+/* head_dim 256 / 512 on the matrix cores (rows 16-byte aligned). 512 with at least 32 keys (the VAE's call; key mask
+ * and causal limit included) takes the kernel in which a wave owns 32 whole queries; its key ranges, if it cuts any,
+ * leave their partial results in private scratch, and so does its packed key mask. Everything else takes the kernel
+ * that slices the head dim over the waves. Returns 0 or a HIP error; -1 when the scratch could not be had (already
+ * reported). */
 static int attention_wide(const char *what, const char *name512, const char *name_sliced, uint16_t *out, int ldo,
                           const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi, int seq_q, int seq_k,
                           int heads, int kv_heads, int head_dim, float scale, int causal, const int *key_mask) {
-    if (head_dim == 512 && !causal && !key_mask && seq_k >= 32) {          /* its key tiles are 32 whole rows */
+    if (head_dim == 512 && seq_k >= 32) {          /* its key tiles are 32 whole rows */
         int splits = 1;
-        const size_t need = iris_hip_fa_hd512_plan(seq_q, seq_k, heads, &splits);
+        const size_t need = iris_hip_fa_hd512_plan(seq_q, seq_k, heads, causal != 0, key_mask != NULL, &splits);
         if (need && !scratch_fit(&g_split, &g_split_bytes, need, what)) return -1;
         g_last_kernel = name512;
-        return iris_hip_fa_hd512(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, splits, g_split);
+        return iris_hip_fa_hd512(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal != 0, key_mask, splits,
+                                 g_split);
     }
     g_last_kernel = name_sliced;
     return iris_hip_fa_sliced(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, head_dim, scale, causal != 0,
