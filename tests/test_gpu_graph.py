@@ -152,10 +152,12 @@ def test_double_stream_step_replayed_from_a_graph():
     dev.free_all()
 
 
-def test_head_dim_512_attention_with_key_ranges_replayed_from_a_graph():
-    """The VAE's attention call at 4096 tokens: two launches (key ranges, then their merge through private scratch).
-    Once the scratch exists the call is captured; every replay, with eager calls of another size between them that
-    overwrite the same scratch, equals the eager result."""
+@pytest.mark.parametrize("causal_and_masked", [False, True], ids=["plain", "causal-masked"])
+def test_head_dim_512_attention_with_key_ranges_replayed_from_a_graph(causal_and_masked):
+    """The VAE's attention call at 4096 tokens: two launches (key ranges, then their merge through private scratch), and
+    with a key mask a third in front that packs the mask into the same scratch. Once the scratch exists the call is
+    captured; every replay, with eager calls of another size between them that overwrite the same scratch, equals
+    the eager result."""
     import oracle as O
     dev, g = Dev(), Graphs()
     lib, stream = dev.lib, _vp(dev.lib.iris_dev_stream())
@@ -164,8 +166,10 @@ def test_head_dim_512_attention_with_key_ranges_replayed_from_a_graph():
     buf = O.f32_to_bf16(rng.standard_normal((seq, 3 * hd)).astype(np.float32))
     rows, out, other = dev.put(buf), dev.alloc(seq * hd * 2), dev.alloc(seq * hd * 2)
     scale = float(1 / np.sqrt(hd))
-    args = (out, hd, rows, ptr_add(rows, 2 * hd), ptr_add(rows, 4 * hd), 3 * hd, seq, seq, 1, 1, hd, scale, 0, None)
-    small = (other, hd, rows, ptr_add(rows, 2 * hd), ptr_add(rows, 4 * hd), 3 * hd, 1000, 1000, 1, 1, hd, scale, 0, None)
+    causal = int(causal_and_masked)
+    mask = dev.put((rng.random(seq) < 0.7).astype(np.int32)) if causal_and_masked else None
+    args = (out, hd, rows, ptr_add(rows, 2 * hd), ptr_add(rows, 4 * hd), 3 * hd, seq, seq, 1, 1, hd, scale, causal, mask)
+    small = (other, hd, rows, ptr_add(rows, 2 * hd), ptr_add(rows, 4 * hd), 3 * hd, 1000, 1000, 1, 1, hd, scale, causal, mask)
     lib.iris_dev_attention(*args)                                   # outside: the scratch is sized
     dev.check()
     assert dev.dev.last_kernel() == "fa_hd512"
