@@ -68,9 +68,10 @@ void iris_dev_head_norm_rope(uint16_t *x, int ld, const float *w,
  * and 512 on 16-byte aligned rows run on the matrix cores directly, any other head_dim <= 512 or
  * alignment through a padded, aligned private copy of q, k, v; the rest (head_dim > 512,
  * scale <= 0, more than 250000 masked keys) on a scalar kernel. head_dim 512 with at least 32 keys
- * (the VAE's call, reference iris_vae.c:1112-1124) may cut the keys into ranges whose partial
- * results pass through private scratch (67 MB at 16384 tokens), and keeps a packed copy of the key
- * mask there (4 bytes per 32 keys); every other directly taken layout allocates nothing.
+ * (the VAE's call, reference iris_vae.c:1112-1124) and head_dim 256 may cut the keys into ranges
+ * whose partial results pass through private scratch (67 MB at 16384 tokens x 512), and keep a
+ * packed copy of the key mask there (4 bytes per 32 keys); every other directly taken layout
+ * allocates nothing.
  * Numerics: P = exp(s - max) is rounded to bf16 for the P V product, as in the reference's GPU
  * kernels (iris_cuda.cu:656-665), and the row sum in the denominator is taken over those ROUNDED
  * values (on the matrix cores), where the reference sums the unrounded f32 values (:659-665): the

@@ -50,6 +50,9 @@
  * front); the walk over the keys ends at the last tile that has a valid key.
  * A causal call walks the tiles in front of each workgroup's last query; its
  * workgroups differ in length and are numbered by falling length.
+ *
+ * head_dim 256 is the same kernel with half the k-steps, dim blocks and tile
+ * rows (template parameter HD); the description above gives the numbers of 512.
  */
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -66,13 +69,12 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int HD = 512;
 constexpr int BN = 32;              /* keys per tile */
 constexpr int BM = 128;             /* queries per workgroup */
 constexpr int THREADS = 256;
-constexpr int TILE = BN * HD;       /* elements of a K (or V) tile: 32 KB */
 constexpr int XCDS = 8;
-constexpr size_t LDS_BYTES = 5 * (size_t)TILE * sizeof(uint16_t);      /* three K stages, two V stages: all 160 KB */
+/* three K stages, two V stages of 32 keys x HD: all 160 KB at head_dim 512 */
+constexpr size_t lds_bytes(int hd) { return 5 * (size_t)BN * hd * sizeof(uint16_t); }
 constexpr float RESCALE_THRESHOLD = 8.0f;   /* log2 units */
 
 /* Every lambda below is inlined by the always-inline pass, before anything else runs: a closure that is only
@@ -110,7 +112,7 @@ __device__ __forceinline__ const uint16_t *scalar_ptr(const uint16_t *p) {
     return (const uint16_t *)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
 
-/* Where the partial results of a key range live: [range][head][query] rows of 512 f32, and (max, sum) pairs. */
+/* Where the partial results of a key range live: [range][head][query] rows of HD f32, and (max, sum) pairs. */
 struct Partials {
     float *o, *ml;
 };
@@ -137,16 +139,22 @@ __host__ inline int causal_pairs(int q_tiles, int step, int splits) {
     return n;
 }
 
-/* SPLIT: one of several key ranges (partial results to `part`). CAUSAL: query i ignores keys j > i; a workgroup walks
+/* HD: 512, or 256 (the same kernel with half the k-steps, dim blocks and tile rows: a tile row is then half of what one
+ * load instruction moves, and a wave's eight rows of a tile are four instructions of two rows). SPLIT: one of several
+ * key ranges (partial results to `part`). CAUSAL: query i ignores keys j > i; a workgroup walks
  * the tiles of its range up to its last query, and the workgroups are numbered by falling length. MASK:
  * `mask_words[t]` holds the valid keys of key tile t as k_pack_key_mask left them. */
-template <bool SPLIT, bool CAUSAL, bool MASK>
+template <int HD, bool SPLIT, bool CAUSAL, bool MASK>
 __global__ void __launch_bounds__(THREADS, 1)
 k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__ q,
                const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int ldi,
                int seq_q, int seq_k, int heads, int q_tiles, int splits, int tiles_per_split,
                int total_work, int work_per_xcd, int kv_group, float scale_log2, Partials part,
                const uint32_t *__restrict__ mask_words) {
+    static_assert(HD == 512 || HD == 256, "rows of one or half a load instruction");
+    constexpr int TILE = BN * HD;                       /* elements of a K (or V) tile */
+    constexpr int KS = HD / 32, DB = HD / 16;           /* k-steps of the score products, dim blocks of the output */
+    constexpr int RPI = 512 / HD, NR = 8 / RPI;         /* tile rows per load instruction; instructions per wave and tile */
     extern __shared__ __align__(16) uint16_t lds[];     /* K stages 0, 1, 2 | V stages 0, 1 */
 
     int qt, split, head;
@@ -232,16 +240,20 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             v_rd[i] = 3 * TILE + vrow * HD + 8 * ((2 * i + ((li & 3) >> 1)) ^ swz(vrow)) + 4 * (li & 1);
     }
 
-    /* One tile row (1 KB) per instruction: lane i fills slot i of row r = 8 wave + j of the stage, i.e. fetches chunk
-     * i ^ swz(r) = i ^ 2 j of global row r. A wave's eight rows of a tile differ in the per-lane offset only (row j:
-     * j row strides further), kept in eight registers, so that a request is three instructions: M0, a wait state,
-     * the load, with one scalar source pointer per tile. A tile never reaches past the last key: the last tile of a
+    /* 1 KB per instruction, one tile row at head_dim 512: lane i fills slot i of row r = 8 wave + j of the stage, i.e.
+     * fetches chunk i ^ swz(r) = i ^ 2 j of global row r (two rows at head_dim 256: lanes 0-31 row 8 wave + 2 j, lanes
+     * 32-63 the next, 32 slots each). A wave's rows of a tile differ in the per-lane offset only (row j: j row
+     * strides further), kept in NR registers, so that a request is three instructions: M0, a wait state, the load,
+     * with one scalar source pointer per tile. A tile never reaches past the last key: the last tile of a
      * sequence whose length is not a multiple of 32 is moved back to end with it, and the keys it then shares
      * with the tile before are masked there (seq_k >= 32). Tiles past the end of the range repeat its last tile.
      * `stage` counts TILEs from the start of the LDS. */
-    uint32_t lane_off[8];
+    uint32_t lane_off[NR];
 #pragma unroll
-    for (int j = 0; j < 8; j++) lane_off[j] = ((16u * (uint32_t)lane) ^ (32u * (uint32_t)j)) + (uint32_t)j * (uint32_t)ldi * 2u;
+    for (int j = 0; j < NR; j++) {
+        const uint32_t row = (uint32_t)(RPI * j + (RPI == 2 ? lane >> 5 : 0)), slot = (uint32_t)(lane & (64 / RPI - 1));
+        lane_off[j] = 16u * (slot ^ (2u * (row & 7u))) + row * (uint32_t)ldi * 2u;
+    }
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds)) + (uint32_t)(8 * wave * HD * 2);
     auto tile_rows = [&](const uint16_t *base, int tile) INLINE {          /* the wave's first row of a tile of the range */
         const int k0 = min((t_begin + min(tile, nt - 1)) * BN, seq_k - BN);
@@ -250,16 +262,16 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     auto request_row = [&](const uint16_t *rows, int stage, int j) INLINE {
         const uint32_t dst = lds0 + (uint32_t)(stage * TILE * 2);
         asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
-                     ::"s"(dst), "n"(j * HD * 2), "v"(lane_off[j]), "s"(rows) : "memory", "m0", "scc");
+                     ::"s"(dst), "n"(j * 1024), "v"(lane_off[j]), "s"(rows) : "memory", "m0", "scc");
     };
 
-    f32x4 o[32][2];                                  /* O^T: dims 16 db + 4 lg + r of query block nb */
+    f32x4 o[DB][2];                                  /* O^T: dims 16 db + 4 lg + r of query block nb */
     float m_run[2], neg_m[2], bound[2];
     f32x4 l_acc[2];
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
 #pragma unroll
-        for (int db = 0; db < 32; db++) {
+        for (int db = 0; db < DB; db++) {
             o[db][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             asm volatile("" : "+a"(o[db][nb]));
         }
@@ -278,22 +290,22 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     {
         const uint16_t *k0r = tile_rows(kbase, 0), *v0r = tile_rows(vbase, 0), *k1r = tile_rows(kbase, 1), *k2r = tile_rows(kbase, 2);
 #pragma unroll
-        for (int j = 0; j < 8; j++) request_row(k0r, 0, j);
+        for (int j = 0; j < NR; j++) request_row(k0r, 0, j);
 #pragma unroll
-        for (int j = 0; j < 8; j++) request_row(v0r, 3, j);
+        for (int j = 0; j < NR; j++) request_row(v0r, 3, j);
 #pragma unroll
-        for (int j = 0; j < 8; j++) request_row(k1r, 1, j);
+        for (int j = 0; j < NR; j++) request_row(k1r, 1, j);
 #pragma unroll
-        for (int j = 0; j < 8; j++) request_row(k2r, 2, j);
+        for (int j = 0; j < NR; j++) request_row(k2r, 2, j);
     }
 
     /* Q^T as B operands: for query block nb and k-step ks the lane holds dims 32 ks + 8 lg .. +7 of query 16 nb + li */
-    bf16x8 qb[2][16];
+    bf16x8 qb[2][KS];
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
         const uint16_t *qp = q + (size_t)min(qrow0 + 16 * nb, seq_q - 1) * ldi + (size_t)head * HD + 8 * lg;
 #pragma unroll
-        for (int ks = 0; ks < 16; ks++)
+        for (int ks = 0; ks < KS; ks++)
             qb[nb][ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(qp + 32 * ks));
     }
     /* the tile requests are invisible to the compiler's wait-count bookkeeping: complete the loads it knows about
@@ -301,7 +313,7 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 #pragma unroll
     for (int nb = 0; nb < 2; nb++)
 #pragma unroll
-        for (int ks = 0; ks < 16; ks++) {
+        for (int ks = 0; ks < KS; ks++) {
             u32x4 t = __builtin_bit_cast(u32x4, qb[nb][ks]);
             asm volatile("" : "+v"(t));
             qb[nb][ks] = __builtin_bit_cast(bf16x8, t);
@@ -309,7 +321,8 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
     wait_vmcnt<0>();
     lds_barrier();
 
-    /* ---- S^T = K Q^T of one tile into s: 2 key blocks x 2 query blocks, 16 k-steps of 32 dims. A wave that is
+    /* ---- S^T = K Q^T of one tile into s: 2 key blocks x 2 query blocks, 16 k-steps of 32 dims (the numbers in these
+     * comments are those of head_dim 512; 256 has half the k-steps, dim blocks and requests). A wave that is
      * alone on its SIMD issues in order, and what it issues between two products runs while the matrix core works on
      * the first: one memory instruction per gap is free, more are not. So the two operand reads of k-step ks + KD
      * stand behind the first and the third product of k-step ks, and between(i) behind the i-th of the 64 products
@@ -325,14 +338,14 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         for (int ks = 0; ks < KD; ks++) { read_k(ks, 0); read_k(ks, 1); }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int ks = 0; ks < 16; ks++) {
+        for (int ks = 0; ks < KS; ks++) {
 #pragma unroll
             for (int mb = 0; mb < 2; mb++)
 #pragma unroll
                 for (int nb = 0; nb < 2; nb++) {
                     if (ks == 0) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=&v"(s[mb][nb]) : "v"(ka[0][mb]), "v"(qb[nb][0]));
                     else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(s[mb][nb]) : "v"(ka[ks % (KD + 1)][mb]), "v"(qb[nb][ks]));
-                    if (nb == 0 && ks + KD < 16) read_k(ks + KD, mb);
+                    if (nb == 0 && ks + KD < KS) read_k(ks + KD, mb);
                     between(4 * ks + 2 * mb + nb);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -400,7 +413,7 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                 asm volatile("" : "+v"(l_acc[nb]));
                 l_acc[nb] *= alpha;
 #pragma unroll
-                for (int db = 0; db < 32; db++) {
+                for (int db = 0; db < DB; db++) {
                     asm volatile("" : "+a"(o[db][nb]));
                     f32x4 t = o[db][nb];
                     t *= alpha;
@@ -443,14 +456,14 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         for (int nb = 0; nb < 2; nb++)
             asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(l_acc[nb]) : "v"(ones), "v"(pw[nb]));
 #pragma unroll
-        for (int g = 0; g < 16; g++) {
+        for (int g = 0; g < DB / 2; g++) {
 #pragma unroll
             for (int d = 0; d < 2; d++) {
                 const s16x8 both = __builtin_shufflevector(lo[g % (VD + 1)][d], hi[g % (VD + 1)][d], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
                 for (int nb = 0; nb < 2; nb++) {
                     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(o[2 * g + d][nb]) : "v"(both), "v"(pw[nb]));
-                    if (g + VD < 16) read_v(g + VD, 2 * d + nb);
+                    if (g + VD < DB / 2) read_v(g + VD, 2 * d + nb);
                     between(4 * g + 2 * d + nb);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -502,7 +515,7 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         kstage = kstage == 2 ? 0 : kstage + 1;
 #pragma unroll
         for (int i = 0; i < 4; i++) k_cur[i] += step;
-        wait_vmcnt<8>();
+        wait_vmcnt<NR>();
         lds_barrier();
     };
     for (int t = 0; t < nt; t += 2) {
@@ -515,7 +528,7 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
 #pragma unroll
-        for (int db = 0; db < 32; db++) asm volatile("" : "+a"(o[db][nb]));
+        for (int db = 0; db < DB; db++) asm volatile("" : "+a"(o[db][nb]));
         asm volatile("" : "+v"(l_acc[nb]));
     }
 
@@ -529,13 +542,13 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
             const size_t prow = ((size_t)split * heads + head) * seq_q + qrow;
             float *po = part.o + prow * HD + 4 * lg;
 #pragma unroll
-            for (int db = 0; db < 32; db++) *reinterpret_cast<f32x4 *>(po + 16 * db) = o[db][nb];
+            for (int db = 0; db < DB; db++) *reinterpret_cast<f32x4 *>(po + 16 * db) = o[db][nb];
             if (lg == 0) *reinterpret_cast<f32x2 *>(part.ml + 2 * prow) = f32x2{m_run[nb], l_tot};
         } else {
             const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
             uint16_t *op = out + (size_t)qrow * ldo + (size_t)head * HD + 4 * lg;
 #pragma unroll
-            for (int db = 0; db < 32; db++) {
+            for (int db = 0; db < DB; db++) {
                 uint2 w;
                 w.x = pack_bf16(o[db][nb][0] * inv, o[db][nb][1] * inv);
                 w.y = pack_bf16(o[db][nb][2] * inv, o[db][nb][3] * inv);
@@ -563,7 +576,8 @@ k_pack_key_mask(uint32_t *__restrict__ words, const int *__restrict__ key_mask, 
 }
 
 /* Combines the key ranges of a query: out = sum_r 2^(m_r - m) o_r / sum_r 2^(m_r - m) l_r with m the largest of the
- * maxima. 64 threads per query row, 8 dims each. */
+ * maxima. 64 threads per query row, HD / 64 dims each. */
+template <int HD>
 __global__ void __launch_bounds__(256)
 k_fa_hd512_merge(uint16_t *__restrict__ out, int ldo, Partials part, int seq_q, int heads, int splits, int causal_keys,
                  int tiles_per_split) {
@@ -578,21 +592,28 @@ k_fa_hd512_merge(uint16_t *__restrict__ out, int ldo, Partials part, int seq_q, 
     }
     float m = -INFINITY;
     for (int r = 0; r < splits; r++) m = fmaxf(m, part.ml[2 * (r * rows + row)]);
+    constexpr int PER = HD / 64;                      /* 8 or 4 */
     float l = 0.0f, acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     for (int r = 0; r < splits; r++) {
         const f32x2 ml = *reinterpret_cast<const f32x2 *>(part.ml + 2 * (r * rows + row));
         if (ml[0] == -INFINITY) continue;             /* no valid key in this range */
         const float w = __builtin_amdgcn_exp2f(ml[0] - m);
         l += w * ml[1];
-        const float *po = part.o + (r * rows + row) * HD + 8 * t;
-        const f32x4 a = *reinterpret_cast<const f32x4 *>(po), b = *reinterpret_cast<const f32x4 *>(po + 4);
+        const float *po = part.o + (r * rows + row) * HD + PER * t;
+        const f32x4 a = *reinterpret_cast<const f32x4 *>(po);
 #pragma unroll
-        for (int i = 0; i < 4; i++) { acc[i] += w * a[i]; acc[4 + i] += w * b[i]; }
+        for (int i = 0; i < 4; i++) acc[i] += w * a[i];
+        if (PER == 8) {
+            const f32x4 b = *reinterpret_cast<const f32x4 *>(po + 4);
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[4 + i] += w * b[i];
+        }
     }
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    uint16_t *op = out + qrow * ldo + head * HD + 8 * t;                  /* output rows are 8-byte aligned, not more */
+    uint16_t *op = out + qrow * ldo + head * HD + PER * t;                /* output rows are 8-byte aligned, not more */
     *reinterpret_cast<uint2 *>(op) = make_uint2(pack_bf16(acc[0] * inv, acc[1] * inv), pack_bf16(acc[2] * inv, acc[3] * inv));
-    *reinterpret_cast<uint2 *>(op + 4) = make_uint2(pack_bf16(acc[4] * inv, acc[5] * inv), pack_bf16(acc[6] * inv, acc[7] * inv));
+    if (PER == 8)
+        *reinterpret_cast<uint2 *>(op + 4) = make_uint2(pack_bf16(acc[4] * inv, acc[5] * inv), pack_bf16(acc[6] * inv, acc[7] * inv));
 }
 
 int cu_count() {
@@ -614,19 +635,22 @@ int cu_count() {
 
 /* How many key ranges a call is cut into, and the scratch it then needs (partial rows for more than one range, the
  * packed key mask for a masked call; 0 for neither). Host arithmetic only.
- * Fitted to every number of ranges at 256 .. 50176 tokens: a turn of 32 keys takes a workgroup 1.6 us when all CUs
- * are busy and 1.3 us when few are (the clock follows the load), a round of workgroups costs its turns plus about
- * 8 us of start and end, and the merge reads and writes the partial rows at about 6 TB/s (they are still in the
- * caches) behind a launch of 4 us and half a microsecond per range. The choice is within 3 % of the best count from
- * 9216 tokens on and within 6 % below (where every count from 4 to 8 is within 10 % of every other).
+ * Fitted at head_dim 512 to every number of ranges at 256 .. 50176 tokens: a turn of 32 keys takes a workgroup 1.6 us
+ * when all CUs are busy and 1.3 us when few are (the clock follows the load), a round of workgroups costs its turns
+ * plus about 8 us of start and end, and the merge reads and writes the partial rows at about 6 TB/s (they are still
+ * in the caches) behind a launch of 4 us and half a microsecond per range. The choice is within 3 % of the best
+ * count from 9216 tokens on and within 6 % below (where every count from 4 to 8 is within 10 % of every other).
  * A causal call has workgroups of 4, 8, 12, ... tiles: it takes the longer of its longest workgroup and of all its
  * turns spread over the CUs, and ranges shorten the former; ranges that begin behind a workgroup's last query do
  * not exist, in the kernel and in the merge. Fitted to 1 .. 8 ranges at 1024 .. 30000 tokens: the choice costs 1 %
- * on average against the best count. */
-extern "C" size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int causal, int masked, int *splits_out) {
+ * on average against the best count. At head_dim 256 a turn has half the products and costs TURN_256 of the above. */
+namespace {
+constexpr double TURN_256 = 0.6;
+size_t plan_ranges(int hd, int seq_q, int seq_k, int heads, int causal, int masked, int *splits_out) {
     const long cus = cu_count();
     const long tiles = (seq_k + BN - 1) / BN, q_tiles = (seq_q + BM - 1) / BM, wgs = q_tiles * heads;
-    const double rows_mb = (double)seq_q * heads * HD * 4 / 1e6;          /* one range's partial O, MB */
+    const double rows_mb = (double)seq_q * heads * hd * 4 / 1e6;          /* one range's partial O, MB */
+    const double turn = hd == 512 ? 1.0 : TURN_256;
     double best = 0.0;
     int best_s = 1;
     for (int s = 1; s <= 8 && s <= tiles; s++) {
@@ -644,12 +668,12 @@ extern "C" size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int ca
              * end; a turn costs 1.2 us on an empty machine and 1.7 us on a full one */
             const double longest = (double)(per < tiles ? per : tiles), spread = (double)turns * heads / cus + 0.2 * longest;
             const double span = filled * heads <= cus || longest > spread ? longest : spread;
-            us = span * (1.2 + 0.5 * (double)turns * heads / (cus * span)) + 10.0 * (double)((filled * heads + cus - 1) / cus);
-            if (ranges > 1) us += 4.0 + 0.5 * ranges + 2.0 * (double)filled * heads * (BM * HD * 4 / 1e6) / 6.0;
+            us = span * turn * (1.2 + 0.5 * (double)turns * heads / (cus * span)) + 10.0 * (double)((filled * heads + cus - 1) / cus);
+            if (ranges > 1) us += 4.0 + 0.5 * ranges + 2.0 * (double)filled * heads * (BM * hd * 4 / 1e6) / 6.0;
         } else {
             const long full = wgs * ranges / cus, rest = wgs * ranges % cus;
-            us = full * (per * 1.6 + 8.0);
-            if (rest) us += per * (1.3 + 0.3 * (double)rest / cus) + 8.0;
+            us = full * (per * turn * 1.6 + 8.0);
+            if (rest) us += per * turn * (1.3 + 0.3 * (double)rest / cus) + 8.0;
             if (ranges > 1) us += 4.0 + 0.5 * ranges + 2.0 * ranges * rows_mb / 6.0;          /* MB / (TB/s) = us */
         }
         if (s == 1 || us < best * 0.97) { best = us; best_s = s; }
@@ -657,7 +681,15 @@ extern "C" size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int ca
     *splits_out = best_s;
     const size_t rows = best_s == 1 ? 0 : (size_t)seq_q * heads * best_s;
     const size_t words = masked ? ((size_t)tiles + 2) / 2 * 2 : 0;
-    return rows * HD * sizeof(float) + rows * 2 * sizeof(float) + words * sizeof(uint32_t);
+    return rows * hd * sizeof(float) + rows * 2 * sizeof(float) + words * sizeof(uint32_t);
+}
+}  // namespace
+
+extern "C" size_t iris_hip_fa_hd512_plan(int seq_q, int seq_k, int heads, int causal, int masked, int *splits_out) {
+    return plan_ranges(512, seq_q, seq_k, heads, causal, masked, splits_out);
+}
+extern "C" size_t iris_hip_fa_hd256_plan(int seq_q, int seq_k, int heads, int causal, int masked, int *splits_out) {
+    return plan_ranges(256, seq_q, seq_k, heads, causal, masked, splits_out);
 }
 
 /* The numbering of a causal call's workgroups, for inspection on the host: pair `number` of a call with q_tiles query
@@ -673,35 +705,29 @@ extern "C" int iris_hip_fa_hd512_causal_order(int number, int q_tiles, int tiles
 }
 
 namespace {
-template <bool SPLIT, bool CAUSAL, bool MASK>
-int launch_hd512(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi,
-                 int seq_q, int seq_k, int heads, int kv_heads, float scale, int splits, int per, Partials part,
-                 const uint32_t *mask_words) {
+template <int HD, bool SPLIT, bool CAUSAL, bool MASK>
+int launch_wide(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi,
+                int seq_q, int seq_k, int heads, int kv_heads, float scale, int splits, int per, Partials part,
+                const uint32_t *mask_words) {
     static bool configured = false;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd512<SPLIT, CAUSAL, MASK>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_BYTES);
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fa_fwd_hd512<HD, SPLIT, CAUSAL, MASK>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(HD));
         if (e != hipSuccess) return (int)e;
         configured = true;
     }
     const int q_tiles = (seq_q + BM - 1) / BM;
     const int total = (CAUSAL ? causal_pairs(q_tiles, per / 4, splits) : q_tiles * splits) * heads;
     const int per_xcd = CAUSAL ? (total + 31) / 32 * 4 : (total + XCDS - 1) / XCDS;     /* causal: whole groups of 32 */
-    hipLaunchKernelGGL((k_fa_fwd_hd512<SPLIT, CAUSAL, MASK>), dim3(per_xcd * XCDS), dim3(THREADS), LDS_BYTES, st, out, ldo, q, k, v,
-                       ldi, seq_q, seq_k, heads, q_tiles, splits, per, total, per_xcd, heads / kv_heads,
+    hipLaunchKernelGGL((k_fa_fwd_hd512<HD, SPLIT, CAUSAL, MASK>), dim3(per_xcd * XCDS), dim3(THREADS), lds_bytes(HD), st, out, ldo,
+                       q, k, v, ldi, seq_q, seq_k, heads, q_tiles, splits, per, total, per_xcd, heads / kv_heads,
                        scale * 1.4426950408889634f, part, mask_words);
     return (int)hipGetLastError();
 }
-}  // namespace
 
-/* head_dim 512; rows 16-byte aligned (ldi % 8 == 0, ldo % 4 == 0), seq_k >= 32, scale > 0; key_mask: device int
- * [seq_k] or null. `splits` and `scratch` (16-byte aligned) as iris_hip_fa_hd512_plan says for the same sizes and
- * flags; scratch may be null when it says 0 bytes. */
-extern "C" int iris_hip_fa_hd512(void *stream, uint16_t *out, int ldo, const uint16_t *q,
-                                 const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
-                                 int seq_k, int heads, int kv_heads, float scale, int causal, const int *key_mask,
-                                 int splits, void *scratch) {
-    hipStream_t st = (hipStream_t)stream;
+template <int HD>
+int fa_wide(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
+            int seq_k, int heads, int kv_heads, float scale, int causal, const int *key_mask, int splits, void *scratch) {
     const int tiles = (seq_k + BN - 1) / BN;
     if (seq_k < BN || splits < 1 || splits > tiles || ((splits > 1 || key_mask) && !scratch))
         return (int)hipErrorInvalidValue;
@@ -716,23 +742,33 @@ extern "C" int iris_hip_fa_hd512(void *stream, uint16_t *out, int ldo, const uin
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
     }
+#define IRIS_WIDE(S, C, M) launch_wide<HD, S, C, M>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, splits, per, part, words)
     int e;
-    if (causal && splits == 1) {
-        e = key_mask ? launch_hd512<false, true, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, 1, per, part, words)
-                     : launch_hd512<false, true, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, 1, per, part, words);
-    } else if (causal) {
-        e = key_mask ? launch_hd512<true, true, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, splits, per, part, words)
-                     : launch_hd512<true, true, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, splits, per, part, words);
-    } else if (splits == 1) {
-        e = key_mask ? launch_hd512<false, false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, 1, per, part, words)
-                     : launch_hd512<false, false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, 1, per, part, words);
-    } else {
-        e = key_mask ? launch_hd512<true, false, true>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, splits, per, part, words)
-                     : launch_hd512<true, false, false>(st, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, splits, per, part, words);
-    }
+    if (splits == 1) e = causal ? (key_mask ? IRIS_WIDE(false, true, true) : IRIS_WIDE(false, true, false))
+                                : (key_mask ? IRIS_WIDE(false, false, true) : IRIS_WIDE(false, false, false));
+    else e = causal ? (key_mask ? IRIS_WIDE(true, true, true) : IRIS_WIDE(true, true, false))
+                    : (key_mask ? IRIS_WIDE(true, false, true) : IRIS_WIDE(true, false, false));
+#undef IRIS_WIDE
     if (e || splits == 1) return e;
     const size_t merge_rows = (size_t)seq_q * heads;
-    hipLaunchKernelGGL(k_fa_hd512_merge, dim3((unsigned)((merge_rows + 3) / 4)), dim3(256), 0, st, out, ldo, part, seq_q,
+    hipLaunchKernelGGL(k_fa_hd512_merge<HD>, dim3((unsigned)((merge_rows + 3) / 4)), dim3(256), 0, st, out, ldo, part, seq_q,
                        heads, splits, causal ? seq_k : 0, per);
     return (int)hipGetLastError();
+}
+}  // namespace
+
+/* head_dim 512 (or 256); rows 16-byte aligned (ldi % 8 == 0, ldo % 4 == 0), seq_k >= 32, scale > 0; key_mask: device
+ * int [seq_k] or null. `splits` and `scratch` (16-byte aligned) as the plan function of the same head_dim says for the
+ * same sizes and flags; scratch may be null when it says 0 bytes. */
+extern "C" int iris_hip_fa_hd512(void *stream, uint16_t *out, int ldo, const uint16_t *q,
+                                 const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
+                                 int seq_k, int heads, int kv_heads, float scale, int causal, const int *key_mask,
+                                 int splits, void *scratch) {
+    return fa_wide<512>((hipStream_t)stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, splits, scratch);
+}
+extern "C" int iris_hip_fa_hd256(void *stream, uint16_t *out, int ldo, const uint16_t *q,
+                                 const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
+                                 int seq_k, int heads, int kv_heads, float scale, int causal, const int *key_mask,
+                                 int splits, void *scratch) {
+    return fa_wide<256>((hipStream_t)stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal, key_mask, splits, scratch);
 }

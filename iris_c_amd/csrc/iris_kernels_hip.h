@@ -82,6 +82,11 @@ int iris_hip_fa_hd512_causal_order(int number, int q_tiles, int tiles_per_split,
 int iris_hip_fa_hd512(void *stream, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
                       const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads,
                       float scale, int causal, const int *key_mask, int splits, void *scratch);
+/* the same kernel at head_dim 256 (half the products per tile of 32 keys), with its own plan */
+size_t iris_hip_fa_hd256_plan(int seq_q, int seq_k, int heads, int causal, int masked, int *splits);
+int iris_hip_fa_hd256(void *stream, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k,
+                      const uint16_t *v, int ldi, int seq_q, int seq_k, int heads, int kv_heads,
+                      float scale, int causal, const int *key_mask, int splits, void *scratch);
 
 /* Any head_dim (up to IRIS_ATTENTION_Q_IN_LDS_MAX_HEAD_DIM the 8 queries of a workgroup are kept in LDS as f32,
  * beyond it they are read from global memory), any stride / alignment / scale; the rows of q may have a stride

@@ -306,23 +306,28 @@ void iris_dev_head_norm_rope_qk_streams(uint16_t *xq, uint16_t *xk, int ld,
                       split_half);
 }
 
-/* head_dim 256 / 512 on the matrix cores (rows 16-byte aligned). 512 with at least 32 keys (the VAE's call; key mask
- * and causal limit included) takes the kernel in which a wave owns 32 whole queries; its key ranges, if it cuts any,
- * leave their partial results in private scratch, and so does its packed key mask. Everything else takes the kernel
- * that slices the head dim over the waves. Returns 0 or a HIP error; -1 when the scratch could not be had (already
- * reported). */
-static int attention_wide(const char *what, const char *name512, const char *name_sliced, uint16_t *out, int ldo,
+/* head_dim 256 / 512 on the matrix cores (rows 16-byte aligned). With at least 32 keys (the VAE's call at head_dim
+ * 512; key mask and causal limit included) they take the kernel in which a wave owns 32 whole queries; its key
+ * ranges, if it cuts any, leave their partial results in private scratch, and so does its packed key mask. Fewer
+ * keys take the kernel that slices the head dim over the waves. `kind`: 0 direct, 1 through the padded copy, 2 that
+ * with Q normalised. Returns 0 or a HIP error; -1 when the scratch could not be had (already reported). */
+static int attention_wide(const char *what, int kind, uint16_t *out, int ldo,
                           const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi, int seq_q, int seq_k,
                           int heads, int kv_heads, int head_dim, float scale, int causal, const int *key_mask) {
-    if (head_dim == 512 && seq_k >= 32) {          /* its key tiles are 32 whole rows */
+    static const char *const names[3][3] = {{"fa_hd512", "fa_hd512_packed", "fa_hd512_packed_qnorm"},
+                                            {"fa_hd256", "fa_hd256_packed", "fa_hd256_packed_qnorm"},
+                                            {"fa_sliced", "fa_sliced_packed", "fa_sliced_packed_qnorm"}};
+    if (seq_k >= 32) {                             /* its key tiles are 32 whole rows */
         int splits = 1;
-        const size_t need = iris_hip_fa_hd512_plan(seq_q, seq_k, heads, causal != 0, key_mask != NULL, &splits);
+        const size_t need = head_dim == 512 ? iris_hip_fa_hd512_plan(seq_q, seq_k, heads, causal != 0, key_mask != NULL, &splits)
+                                            : iris_hip_fa_hd256_plan(seq_q, seq_k, heads, causal != 0, key_mask != NULL, &splits);
         if (need && !scratch_fit(&g_split, &g_split_bytes, need, what)) return -1;
-        g_last_kernel = name512;
-        return iris_hip_fa_hd512(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal != 0, key_mask, splits,
-                                 g_split);
+        g_last_kernel = names[head_dim == 512 ? 0 : 1][kind];
+        return head_dim == 512
+                   ? iris_hip_fa_hd512(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal != 0, key_mask, splits, g_split)
+                   : iris_hip_fa_hd256(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal != 0, key_mask, splits, g_split);
     }
-    g_last_kernel = name_sliced;
+    g_last_kernel = names[2][kind];
     return iris_hip_fa_sliced(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, head_dim, scale, causal != 0,
                               key_mask);
 }
@@ -376,8 +381,7 @@ static void attention(const char *what, uint16_t *out, int ldo,
     }
     const int mfma_args = seq_k > 0 && scale > 0.0f && head_dim <= 512 && (!key_mask || seq_k <= IRIS_FA_MAX_MASKED_KEYS);
     if (mfma_ok && !wq && (head_dim == 256 || head_dim == 512)) {
-        err = attention_wide(what, "fa_hd512", "fa_sliced", out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, head_dim,
-                             scale, causal, key_mask);
+        err = attention_wide(what, 0, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, head_dim, scale, causal, key_mask);
         if (err < 0) return;
     } else if (mfma_args) {
         /* Any head_dim <= 512, any stride and alignment: q | k | v copied into one fused row buffer with
@@ -399,9 +403,8 @@ static void attention(const char *what, uint16_t *out, int ldo,
                 err = iris_hip_fa_hd128(g_stream, outp, ldout, packed, pk, pv, ldp, seq_q, seq_k, heads, kv_heads,
                                         scale, causal != 0, key_mask);
             } else {
-                err = attention_wide(what, wq ? "fa_hd512_packed_qnorm" : "fa_hd512_packed",
-                                     wq ? "fa_sliced_packed_qnorm" : "fa_sliced_packed", outp, ldout, packed, pk, pv, ldp,
-                                     seq_q, seq_k, heads, kv_heads, hdp, scale, causal, key_mask);
+                err = attention_wide(what, wq ? 2 : 1, outp, ldout, packed, pk, pv, ldp, seq_q, seq_k, heads, kv_heads, hdp,
+                                     scale, causal, key_mask);
                 if (err < 0) return;
             }
         }

@@ -371,8 +371,8 @@ def test_output_stride_and_interior_pointers(dev, orc, fa):
 @pytest.mark.parametrize("seq_q,seq_k,causal,masked", [(150, 150, False, False), (1, 1, False, False), (33, 95, False, True),
                                                          (64, 64, True, False), (257, 257, True, True), (130, 1000, False, False)])
 def test_wide_heads_256_512(dev, orc, hd, heads, kv, seq_q, seq_k, causal, masked):
-    """head_dim 256 / 512 run on the matrix cores too: 512 with at least 32 keys (the VAE's single 512-wide head; with
-    key mask and causal limit too) in the kernel whose waves own whole queries, the rest in the kernel that slices the
+    """head_dim 256 / 512 run on the matrix cores too: with at least 32 keys (the VAE's single 512-wide head; with key
+    mask and causal limit too) in the kernel whose waves own whole queries, with fewer in the kernel that slices the
     head dim over the waves."""
     buf, ldi = random_case(hd + heads + seq_q, seq_q, seq_k, heads, kv, hd=hd)
     qd, kd = heads * hd, kv * hd
@@ -382,7 +382,7 @@ def test_wide_heads_256_512(dev, orc, hd, heads, kv, seq_q, seq_k, causal, maske
         mask[0] = 1                                        # every causal row keeps a valid key
     scale = float(1 / np.sqrt(hd))
     out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
-    assert kernel == ("fa_hd512" if hd == 512 and seq_k >= 32 else "fa_sliced")
+    assert kernel == (f"fa_hd{hd}" if seq_k >= 32 else "fa_sliced")
     want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
     assert_close(O.bf16_to_f32(out[:seq_q]), want, f"wide hd={hd} {seq_q}x{seq_k}")
 
@@ -424,7 +424,7 @@ def test_vae_shape_at_its_largest_50176_tokens(dev, orc):
 
 
 def test_sliced_kernel_empty_rows_and_large_scores(dev, orc):
-    seq, hd = 100, 256
+    seq, hd = 30, 512                                   # fewer than 32 keys: the kernel that slices the head dim
     buf, ldi = random_case(21, seq, seq, 1, 1, hd=hd, sigma=3.0)          # |score| up to ~100
     scale = float(1 / np.sqrt(hd))
     mask = np.ones(seq, np.int32); mask[:10] = 0
@@ -454,7 +454,7 @@ def test_other_head_dims_run_on_the_matrix_cores_through_a_padded_copy(dev, orc,
     scale = 1 / np.sqrt(hd)
     ldo = heads * hd + 3
     out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq, seq, heads, kv, hd, scale, causal, mask, ldo=ldo)
-    wide = "fa_hd512_packed" if hd > 256 else "fa_sliced_packed"
+    wide = "fa_hd512_packed" if hd > 256 else "fa_hd256_packed"
     assert kernel == ("fa_hd128_packed" if hd <= 128 else wide)
     want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq, seq, heads, kv, hd, scale, causal, mask)
     assert_close(O.bf16_to_f32(out[:, :heads * hd]), want, f"padded copy hd={hd}")
@@ -469,7 +469,7 @@ def test_misaligned_rows_run_on_the_matrix_cores_through_an_aligned_copy(dev, or
     qd = heads * hd
     scale = float(1 / np.sqrt(hd))
     out, kernel = dev.attention(buf, ldi, qoff, qoff + qd, qoff + 2 * qd, seq, seq, heads, heads, hd, scale)
-    assert kernel == {128: "fa_hd128_packed", 256: "fa_sliced_packed", 512: "fa_hd512_packed"}[hd]
+    assert kernel == {128: "fa_hd128_packed", 256: "fa_hd256_packed", 512: "fa_hd512_packed"}[hd]
     want = orc.attention_bf16(buf, ldi, qoff, qoff + qd, qoff + 2 * qd, seq, seq, heads, heads, hd, scale)
     assert_close(O.bf16_to_f32(out), want, f"misaligned hd={hd} pad={pad} offset={qoff}")
 

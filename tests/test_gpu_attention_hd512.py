@@ -1,8 +1,8 @@
-"""The head_dim-512 attention kernel (one wave per SIMD owns 32 whole queries; the VAE mid-block call of the
-reference, iris_vae.c:1112-1124, and the same head size with a key mask or a causal limit, which the device
-interface allows) through the C ABI and, for the number of key ranges, through the kernel's own launcher, against
-the fp32 CPU oracle on identical bf16 inputs. Bars as in test_gpu_attention.py.
-The planner test at the end needs no GPU.
+"""The attention kernel for wide heads (one wave per SIMD owns 32 whole queries): head_dim 512 — the VAE mid-block call
+of the reference, iris_vae.c:1112-1124, and the same head size with a key mask or a causal limit, which the device
+interface allows — and head_dim 256, the same kernel with half the products per tile. Through the C ABI and, for the
+number of key ranges, through the kernel's own launcher, against the fp32 CPU oracle on identical bf16 inputs. Bars
+as in test_gpu_attention.py. The planner tests at the end need no GPU.
 """
 import ctypes as C
 import os
@@ -22,9 +22,9 @@ def dev():
     return Dev()
 
 
-def random_case(seed, seq_q, seq_k, heads, kv, sigma=1.0, pad=0):
+def random_case(seed, seq_q, seq_k, heads, kv, sigma=1.0, pad=0, hd=HD):
     rng = np.random.default_rng(seed)
-    ldi = (heads + 2 * kv) * HD + pad
+    ldi = (heads + 2 * kv) * hd + pad
     buf = O.f32_to_bf16(rng.standard_normal((max(seq_q, seq_k), ldi)).astype(np.float32) * sigma)
     return buf, ldi
 
@@ -35,11 +35,12 @@ def sample_rows(seq, n, seed=0):
     return np.unique(np.clip(np.r_[fixed, rng.integers(0, seq, n)], 0, seq - 1)).astype(np.int32)
 
 
-def plan(lib, seq_q, seq_k, heads, causal=False, masked=False):
-    lib.iris_hip_fa_hd512_plan.restype = C.c_size_t
-    lib.iris_hip_fa_hd512_plan.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int)]
+def plan(lib, seq_q, seq_k, heads, causal=False, masked=False, hd=HD):
+    fn = getattr(lib, f"iris_hip_fa_hd{hd}_plan")
+    fn.restype = C.c_size_t
+    fn.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int)]
     splits = C.c_int(0)
-    need = lib.iris_hip_fa_hd512_plan(seq_q, seq_k, heads, int(causal), int(masked), C.byref(splits))
+    need = fn(seq_q, seq_k, heads, int(causal), int(masked), C.byref(splits))
     return splits.value, need
 
 
@@ -48,17 +49,18 @@ def plan(lib, seq_q, seq_k, heads, causal=False, masked=False):
 @pytest.mark.parametrize("seq_q,seq_k,heads,kv", [(1, 1, 1, 1), (7, 33, 1, 1), (128, 32, 1, 1), (129, 31, 2, 1), (64, 45, 1, 1),
                                                   (40, 63, 2, 2), (300, 1000, 2, 2), (1000, 300, 3, 1), (1024, 1024, 1, 1),
                                                   (2500, 2500, 1, 1), (640, 4100, 4, 2), (200, 1027, 1, 1)])
-def test_shapes_against_the_oracle(dev, orc, seq_q, seq_k, heads, kv):
+@pytest.mark.parametrize("hd", [512, 256])
+def test_shapes_against_the_oracle(dev, orc, hd, seq_q, seq_k, heads, kv):
     """Ragged query and key counts (tiles of 32 keys, workgroups of 128 queries), grouped kv heads, and sizes whose
     keys the launcher cuts into one to eight ranges. A key count that is not a multiple of 32 moves the last tile back
     to end with the sequence and masks the keys it then shares with the tile before (33: all but one of them)."""
-    buf, ldi = random_case(seq_q + 3 * seq_k + heads, seq_q, seq_k, heads, kv, pad=8)
-    qd, kd = heads * HD, kv * HD
-    scale = float(1 / np.sqrt(HD))
-    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, HD, scale, ldo=qd + 4, out_col=4)
-    assert kernel == ("fa_hd512" if seq_k >= 32 else "fa_sliced")       # its key tiles are 32 whole rows
-    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, HD, scale)
-    assert_parity(O.bf16_to_f32(out[:, 4:]), want, f"hd512 {seq_q}x{seq_k} heads {heads}/{kv}")
+    buf, ldi = random_case(seq_q + 3 * seq_k + heads, seq_q, seq_k, heads, kv, pad=8, hd=hd)
+    qd, kd = heads * hd, kv * hd
+    scale = float(1 / np.sqrt(hd))
+    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, ldo=qd + 4, out_col=4)
+    assert kernel == (f"fa_hd{hd}" if seq_k >= 32 else "fa_sliced")       # its key tiles are 32 whole rows
+    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale)
+    assert_parity(O.bf16_to_f32(out[:, 4:]), want, f"hd{hd} {seq_q}x{seq_k} heads {heads}/{kv}")
     assert np.all(out[:, :4] == 0x7fc0)                      # nothing written in front of the output columns
 
 
@@ -125,18 +127,19 @@ def assert_parity_where_keys_are_visible(out, want, causal, mask, what):
 @pytest.mark.parametrize("kind", ["random", "sparse", "prefix", "holes"])
 @pytest.mark.parametrize("seq_q,seq_k,heads,kv", [(128, 32, 1, 1), (100, 77, 1, 1), (40, 63, 2, 2), (300, 1000, 2, 1), (1000, 300, 3, 1),
                                                   (1024, 1024, 1, 1), (640, 4100, 2, 2)])
-def test_key_masks_against_the_oracle(dev, orc, kind, seq_q, seq_k, heads, kv):
+@pytest.mark.parametrize("hd", [512, 256])
+def test_key_masks_against_the_oracle(dev, orc, hd, kind, seq_q, seq_k, heads, kv):
     """The key mask reaches the kernel as one word per tile of 32 keys (a pack kernel in front of it); a tile moved back
     to end with the sequence has the keys it shares with its neighbour cleared there. Masks that leave tiles whole,
     empty or ragged; a mask that leaves no key at all gives zero rows."""
-    buf, ldi = random_case(7 * seq_q + seq_k, seq_q, seq_k, heads, kv)
-    qd, kd = heads * HD, kv * HD
-    scale = float(1 / np.sqrt(HD))
+    buf, ldi = random_case(7 * seq_q + seq_k, seq_q, seq_k, heads, kv, hd=hd)
+    qd, kd = heads * hd, kv * hd
+    scale = float(1 / np.sqrt(hd))
     mask = key_mask_of(kind, seq_k)
-    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, HD, scale, False, mask)
-    assert kernel == "fa_hd512"
-    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, HD, scale, False, mask)
-    assert_parity(O.bf16_to_f32(out), want, f"hd512 {kind} mask {seq_q}x{seq_k} heads {heads}/{kv}")
+    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, False, mask)
+    assert kernel == f"fa_hd{hd}"
+    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, False, mask)
+    assert_parity(O.bf16_to_f32(out), want, f"hd{hd} {kind} mask {seq_q}x{seq_k} heads {heads}/{kv}")
 
 
 @pytest.mark.gpu
@@ -151,19 +154,20 @@ def test_a_mask_without_any_key_gives_zero_rows(dev):
 @pytest.mark.parametrize("seq_q,seq_k,heads,kv", [(128, 32, 1, 1), (128, 128, 1, 1), (100, 77, 1, 1), (77, 100, 1, 1), (1027, 1027, 1, 1),
                                                   (300, 1000, 2, 1), (1000, 300, 2, 1), (2500, 2500, 1, 1), (513, 999, 3, 3),
                                                   (4100, 4100, 2, 1)])
-def test_causal_calls_against_the_oracle(dev, orc, masked, seq_q, seq_k, heads, kv):
+@pytest.mark.parametrize("hd", [512, 256])
+def test_causal_calls_against_the_oracle(dev, orc, hd, masked, seq_q, seq_k, heads, kv):
     """Query i sees keys 0 .. i: a workgroup walks the key tiles in front of its last query only, the launcher cuts
     the keys into ranges as for the full call (a range behind a workgroup's queries does not exist for it), and
     the workgroups are numbered by falling length. More queries than keys, more keys than queries, and a key mask on
     top (rows whose visible keys are all masked are zero, as in the oracle)."""
-    buf, ldi = random_case(5 * seq_q + seq_k, seq_q, seq_k, heads, kv)
-    qd, kd = heads * HD, kv * HD
-    scale = float(1 / np.sqrt(HD))
+    buf, ldi = random_case(5 * seq_q + seq_k, seq_q, seq_k, heads, kv, hd=hd)
+    qd, kd = heads * hd, kv * hd
+    scale = float(1 / np.sqrt(hd))
     mask = key_mask_of("random", seq_k, seed=1) if masked else None
-    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, HD, scale, True, mask)
-    assert kernel == "fa_hd512"
-    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, HD, scale, True, mask)
-    assert_parity_where_keys_are_visible(out, want, True, mask, f"hd512 causal {seq_q}x{seq_k} heads {heads}/{kv} masked {masked}")
+    out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, True, mask)
+    assert kernel == f"fa_hd{hd}"
+    want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, True, mask)
+    assert_parity_where_keys_are_visible(out, want, True, mask, f"hd{hd} causal {seq_q}x{seq_k} heads {heads}/{kv} masked {masked}")
 
 
 @pytest.mark.gpu
@@ -204,44 +208,46 @@ def test_causal_16384_tokens_sampled_rows(dev, orc):
 @pytest.mark.gpu
 @pytest.mark.parametrize("seed", [1, 2])
 def test_random_shapes(dev, orc, seed):
-    """Seeded random sweep at head_dim 512: 32 .. 1500 keys (ragged against the tiles of 32 keys and, through the
+    """Seeded random sweep at head_dim 512 and 256: 32 .. 1500 keys (ragged against the tiles of 32 keys and, through the
     launcher's choice, against every number of key ranges), 1 .. 700 queries, one to three kv heads with one or two
     query heads each, padded row strides, two scales and two input spreads; a third of the cases causal, a third
     with a key mask."""
     rng = np.random.default_rng(seed)
     for case in range(25):
+        hd = int(rng.choice([512, 256]))
         kv = int(rng.choice([1, 1, 2, 3]))
         heads = kv * int(rng.choice([1, 1, 2]))
         seq_k = int(rng.integers(32, 1500))
         seq_q = seq_k if rng.random() < 0.5 else int(rng.integers(1, 700))
-        qd, kd = heads * HD, kv * HD
+        qd, kd = heads * hd, kv * hd
         ldi = qd + 2 * kd + int(rng.choice([0, 0, 8, 64]))
         buf = O.f32_to_bf16((rng.standard_normal((max(seq_q, seq_k), ldi)) * rng.choice([0.3, 1.0])).astype(np.float32))
-        scale = float(rng.choice([1 / np.sqrt(HD), 0.02]))
+        scale = float(rng.choice([1 / np.sqrt(hd), 0.02]))
         causal = bool(rng.random() < 1 / 3)
         mask = key_mask_of(str(rng.choice(["random", "prefix", "holes"])), seq_k, seed=case) if rng.random() < 1 / 3 else None
-        what = (f"seed {seed} case {case}: q {seq_q} k {seq_k} heads {heads}/{kv} ldi {ldi} scale {scale:.4f} causal {causal} "
-                f"masked {mask is not None} ranges {plan(dev.lib, seq_q, seq_k, heads, causal, mask is not None)[0]}")
-        out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, HD, scale, causal, mask)
-        assert kernel == "fa_hd512", what
-        want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, HD, scale, causal, mask)
+        what = (f"seed {seed} case {case}: hd {hd} q {seq_q} k {seq_k} heads {heads}/{kv} ldi {ldi} scale {scale:.4f} causal {causal} "
+                f"masked {mask is not None} ranges {plan(dev.lib, seq_q, seq_k, heads, causal, mask is not None, hd)[0]}")
+        out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
+        assert kernel == f"fa_hd{hd}", what
+        want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
         assert_parity_where_keys_are_visible(out, want, causal, mask, what)
 
 
 # ------------------------------------------------------------------ every number of key ranges
-def launch_with_ranges(dev, buf, ldi, seq_q, seq_k, heads, kv, scale, splits, causal=False, mask=None):
+def launch_with_ranges(dev, buf, ldi, seq_q, seq_k, heads, kv, scale, splits, causal=False, mask=None, hd=HD):
     lib = dev.lib
-    lib.iris_hip_fa_hd512.restype = C.c_int
-    lib.iris_hip_fa_hd512.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
+    run = getattr(lib, f"iris_hip_fa_hd{hd}")
+    run.restype = C.c_int
+    run.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
                                       C.c_int, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
     lib.iris_dev_stream.restype = C.c_void_p
-    qd, kd = heads * HD, kv * HD
+    qd, kd = heads * hd, kv * hd
     d = dev.put(buf)
     out0 = np.full((seq_q, qd), 0x7fc0, dtype=np.uint16)
     do = dev.put(out0)
-    scratch = dev.alloc(max(16, seq_q * heads * splits * (HD + 2) * 4) + 4 * ((seq_k + 31) // 32 + 2))
+    scratch = dev.alloc(max(16, seq_q * heads * splits * (hd + 2) * 4) + 4 * ((seq_k + 31) // 32 + 2))
     dm = dev.put(np.ascontiguousarray(mask, np.int32)) if mask is not None else None
-    err = lib.iris_hip_fa_hd512(lib.iris_dev_stream(), do, qd, d, ptr_add(d, 2 * qd), ptr_add(d, 2 * (qd + kd)), ldi, seq_q, seq_k,
+    err = run(lib.iris_dev_stream(), do, qd, d, ptr_add(d, 2 * qd), ptr_add(d, 2 * (qd + kd)), ldi, seq_q, seq_k,
                                 heads, kv, scale, int(causal), dm, splits, scratch)
     dev.check()
     out = dev.get(do, out0.shape, np.uint16)
@@ -250,20 +256,21 @@ def launch_with_ranges(dev, buf, ldi, seq_q, seq_k, heads, kv, scale, splits, ca
 
 
 @pytest.mark.gpu
-def test_every_number_of_key_ranges_gives_the_same_rows(dev, orc):
+@pytest.mark.parametrize("hd", [512, 256])
+def test_every_number_of_key_ranges_gives_the_same_rows(dev, orc, hd):
     """1 to 8 ranges on 2 heads x 260 queries x 1500 keys (47 tiles, the last one partly filled, ranges of unequal
     length): each against the oracle, and against the one-range result: the probabilities of a range are rounded to
     bf16 relative to that range's own running max, so the rows differ by rounding noise only, a small fraction of
     a bf16 step of the outputs' spread on average."""
     seq_q, seq_k, heads, kv = 260, 1500, 2, 1
-    buf, ldi = random_case(11, seq_q, seq_k, heads, kv)
-    scale = float(1 / np.sqrt(HD))
-    want = orc.attention_bf16(buf, ldi, 0, heads * HD, (heads + kv) * HD, seq_q, seq_k, heads, kv, HD, scale)
+    buf, ldi = random_case(11, seq_q, seq_k, heads, kv, hd=hd)
+    scale = float(1 / np.sqrt(hd))
+    want = orc.attention_bf16(buf, ldi, 0, heads * hd, (heads + kv) * hd, seq_q, seq_k, heads, kv, hd, scale)
     tiles = (seq_k + 31) // 32
     one = None
     for splits in range(1, 9):
         per = (tiles + splits - 1) // splits
-        err, out = launch_with_ranges(dev, buf, ldi, seq_q, seq_k, heads, kv, scale, splits)
+        err, out = launch_with_ranges(dev, buf, ldi, seq_q, seq_k, heads, kv, scale, splits, hd=hd)
         if (tiles + per - 1) // per != splits:              # this count would leave a range empty: refused, nothing written
             assert err != 0 and np.all(out == 0x7fc0)
             continue
@@ -300,19 +307,20 @@ def test_every_number_of_key_ranges_with_a_padding_mask(dev, orc, valid):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("masked", [False, True])
-def test_every_number_of_key_ranges_of_a_causal_call(dev, orc, masked):
+@pytest.mark.parametrize("hd", [512, 256])
+def test_every_number_of_key_ranges_of_a_causal_call(dev, orc, hd, masked):
     """1 to 8 ranges on 2 heads x 1500 queries x 1500 keys, causal: the pairs (query tile, range) that exist are
     numbered by falling length, the others are neither launched nor merged. Each count against the oracle."""
     seq, heads, kv = 1500, 2, 1
-    buf, ldi = random_case(12, seq, seq, heads, kv)
-    scale = float(1 / np.sqrt(HD))
+    buf, ldi = random_case(12, seq, seq, heads, kv, hd=hd)
+    scale = float(1 / np.sqrt(hd))
     mask = key_mask_of("random", seq, seed=2) if masked else None
-    want = orc.attention_bf16(buf, ldi, 0, heads * HD, (heads + kv) * HD, seq, seq, heads, kv, HD, scale, True, mask)
+    want = orc.attention_bf16(buf, ldi, 0, heads * hd, (heads + kv) * hd, seq, seq, heads, kv, hd, scale, True, mask)
     tiles = (seq + 31) // 32
     ran = 0
     for splits in range(1, 9):
         per = (tiles + splits - 1) // splits
-        err, out = launch_with_ranges(dev, buf, ldi, seq, seq, heads, kv, scale, splits, True, mask)
+        err, out = launch_with_ranges(dev, buf, ldi, seq, seq, heads, kv, scale, splits, True, mask, hd=hd)
         if (tiles + per - 1) // per != splits:
             assert err != 0 and np.all(out == 0x7fc0)
             continue
@@ -329,10 +337,11 @@ def test_planner_never_leaves_a_range_empty():
     rng = np.random.default_rng(0)
     sizes = [(1, 1, 1), (16384, 16384, 1), (4096, 4096, 1), (50176, 50176, 1), (1024, 1024, 1), (128, 33, 1), (300, 255, 5)]
     sizes += [tuple(int(x) for x in (rng.integers(1, 60000), rng.integers(1, 60000), rng.integers(1, 5))) for _ in range(300)]
-    for seq_q, seq_k, heads in sizes:
+    for n, (seq_q, seq_k, heads) in enumerate(sizes):
         for causal in (False, True):
             for masked in (False, True):
-                splits, need = plan(lib, seq_q, seq_k, heads, causal, masked)
+                HD = (512, 256)[n % 2]
+                splits, need = plan(lib, seq_q, seq_k, heads, causal, masked, HD)
                 tiles = (seq_k + 31) // 32
                 per = (tiles + splits - 1) // splits
                 assert 1 <= splits <= min(8, tiles) and (tiles + per - 1) // per == splits, (seq_q, seq_k, heads, splits)

@@ -124,7 +124,7 @@ def test_other_shapes_go_through_the_normalised_copy(dev, orc, hd, ldi_extra, sp
     mask = (rng.random(seq) < 0.8).astype(np.int32); mask[0] = 1
     got, kernel, after = dev.attention_qnorm(buf, ldi, 0, q_dim, q_dim + kv_dim, seq, seq, heads, kv, hd, scale, w,
                                              np.cos(ang), np.sin(ang), 1e-5, split, causal=True, key_mask=mask)
-    assert kernel == ("fa_hd128_packed_qnorm" if hd <= 128 else "fa_sliced_packed_qnorm")
+    assert kernel == ("fa_hd128_packed_qnorm" if hd <= 128 else "fa_hd256_packed_qnorm")
     assert np.array_equal(after, buf)
     ref = buf.copy()
     orc.head_norm_rope_bf16(ref, ldi, w, np.cos(ang), np.sin(ang), seq, heads, hd, 1e-5, split, col0=0)
