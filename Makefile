@@ -18,7 +18,7 @@ HIPFLAGS = -O3 --offload-arch=$(GPU_ARCH) -fPIC -std=c++17 -Xclang -target-featu
 HOSTDEFS = -D__HIP_PLATFORM_AMD__=1
 CFLAGS   = -O2 -fPIC -Wall -Wextra -std=c11 $(HOSTDEFS) -I$(CSRC) -Iinclude -I$(ROCM_HOME)/include
 
-HIP_SRCS = $(CSRC)/qknorm_rope.hip $(CSRC)/fa_fwd_gfx950.hip $(CSRC)/fa_fwd_sliced_gfx950.hip $(CSRC)/fa_fwd_hd512_gfx950.hip $(CSRC)/attn_generic.hip \
+HIP_SRCS = $(CSRC)/qknorm_rope.hip $(CSRC)/fa_fwd_gfx950.hip $(CSRC)/fa_fwd_hd512_gfx950.hip $(CSRC)/attn_generic.hip \
            $(CSRC)/ew_norm_ops.hip $(CSRC)/gemm_conv_gfx950.hip $(CSRC)/rope_tables.hip
 HIP_OBJS = $(HIP_SRCS:.hip=.o)
 HOST_HDRS = include/iris_dev.h include/iris_rope.h $(CSRC)/iris_kernels_hip.h $(CSRC)/iris_rope_internal.h
@@ -33,7 +33,7 @@ PATH_LIB = iris_c_amd/libiris_dev_path.a
 path: $(PATH_LIB)
 $(CSRC)/iris_rocm_path.o: $(CSRC)/iris_rocm.c $(HOST_HDRS)
 	$(CC) $(CFLAGS) -DIRIS_DEV_PATH_ONLY -c $< -o $@
-$(PATH_LIB): $(CSRC)/qknorm_rope.o $(CSRC)/fa_fwd_gfx950.o $(CSRC)/fa_fwd_sliced_gfx950.o $(CSRC)/fa_fwd_hd512_gfx950.o $(CSRC)/attn_generic.o $(CSRC)/iris_rocm_path.o
+$(PATH_LIB): $(CSRC)/qknorm_rope.o $(CSRC)/fa_fwd_gfx950.o $(CSRC)/fa_fwd_hd512_gfx950.o $(CSRC)/attn_generic.o $(CSRC)/iris_rocm_path.o
 	rm -f $@ && ar rcs $@ $^
 # link check: a host program that defines its OWN iris_dev_init / alloc / ... (as the reference's backend object
 # does) next to the archive: no duplicate symbols, the hot-path calls resolve to the archive

@@ -246,18 +246,20 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
      * strides further), kept in NR registers, so that a request is three instructions: M0, a wait state, the load,
      * with one scalar source pointer per tile. A tile never reaches past the last key: the last tile of a
      * sequence whose length is not a multiple of 32 is moved back to end with it, and the keys it then shares
-     * with the tile before are masked there (seq_k >= 32). Tiles past the end of the range repeat its last tile.
+     * with the tile before are masked there; a sequence of fewer than 32 keys is one tile padded with its last key. Tiles past the end of the range repeat its last tile.
      * `stage` counts TILEs from the start of the LDS. */
     uint32_t lane_off[NR];
 #pragma unroll
     for (int j = 0; j < NR; j++) {
         const uint32_t row = (uint32_t)(RPI * j + (RPI == 2 ? lane >> 5 : 0)), slot = (uint32_t)(lane & (64 / RPI - 1));
-        lane_off[j] = 16u * (slot ^ (2u * (row & 7u))) + row * (uint32_t)ldi * 2u;
+        /* a sequence of fewer than 32 keys is one tile whose last rows repeat its last key (they are masked) */
+        const uint32_t in_tile = min(8u * (uint32_t)wave + row, (uint32_t)min(seq_k, BN) - 1u);
+        lane_off[j] = 16u * (slot ^ (2u * (row & 7u))) + in_tile * (uint32_t)ldi * 2u;
     }
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds)) + (uint32_t)(8 * wave * HD * 2);
-    auto tile_rows = [&](const uint16_t *base, int tile) INLINE {          /* the wave's first row of a tile of the range */
-        const int k0 = min((t_begin + min(tile, nt - 1)) * BN, seq_k - BN);
-        return base + (size_t)(k0 + 8 * wave) * ldi;
+    auto tile_rows = [&](const uint16_t *base, int tile) INLINE {          /* the first row of a tile of the range */
+        const int k0 = max(min((t_begin + min(tile, nt - 1)) * BN, seq_k - BN), 0);
+        return base + (size_t)k0 * ldi;
     };
     auto request_row = [&](const uint16_t *rows, int stage, int j) INLINE {
         const uint32_t dst = lds0 + (uint32_t)(stage * TILE * 2);
@@ -362,7 +364,7 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
         /* valid keys of the tile as a wave-uniform set: the last tile of the sequence is moved back by k0 + 32 - seq_k
          * keys, which belong to the tile before; with a key mask the packed word says all of this already */
         uint32_t valid = ~0u;
-        if (k0 + BN > seq_k) valid = ~0u << (k0 + BN - seq_k);
+        if (k0 + BN > seq_k) valid = seq_k < BN ? ~0u >> (BN - seq_k) : ~0u << (k0 + BN - seq_k);
         if (MASK) valid = mask_word;
         if (valid != ~0u) {
             const unsigned mine = valid >> (4 * lg);
@@ -376,7 +378,7 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
                     }
         }
         if (CAUSAL) {
-            const int first = min(k0, seq_k - BN);              /* the key in row 0 of the tile as it was loaded */
+            const int first = max(min(k0, seq_k - BN), 0);      /* the key in row 0 of the tile as it was loaded */
             if (first + BN - 1 > wq0) {                          /* wave-uniform: some key lies behind the wave's first query */
                 const int lim0 = qrow0 - first - 4 * lg;         /* key offset 16 mb + r is valid iff <= lim0 (+ 16 nb) */
 #pragma unroll
@@ -566,8 +568,8 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 __global__ void __launch_bounds__(64)
 k_pack_key_mask(uint32_t *__restrict__ words, const int *__restrict__ key_mask, int seq_k, int tiles) {
     const int tile = 2 * blockIdx.x + (threadIdx.x >> 5), j = threadIdx.x & 31;
-    const int first = min(tile * BN, seq_k - BN), key = first + j;
-    const bool ok = tile < tiles && key >= tile * BN && key_mask[key] != 0;
+    const int first = max(min(tile * BN, seq_k - BN), 0), key = first + j;
+    const bool ok = tile < tiles && key >= tile * BN && key < seq_k && key_mask[key] != 0;
     const unsigned long long both = __ballot(ok);
     if (threadIdx.x == 0) {
         words[2 * blockIdx.x] = (uint32_t)both;
@@ -729,7 +731,7 @@ template <int HD>
 int fa_wide(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi, int seq_q,
             int seq_k, int heads, int kv_heads, float scale, int causal, const int *key_mask, int splits, void *scratch) {
     const int tiles = (seq_k + BN - 1) / BN;
-    if (seq_k < BN || splits < 1 || splits > tiles || ((splits > 1 || key_mask) && !scratch))
+    if (seq_k < 1 || splits < 1 || splits > tiles || ((splits > 1 || key_mask) && !scratch))
         return (int)hipErrorInvalidValue;
     const int per = (tiles + splits - 1) / splits;
     if ((tiles + per - 1) / per != splits) return (int)hipErrorInvalidValue;      /* an empty range */
@@ -757,7 +759,7 @@ int fa_wide(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uin
 }
 }  // namespace
 
-/* head_dim 512 (or 256); rows 16-byte aligned (ldi % 8 == 0, ldo % 4 == 0), seq_k >= 32, scale > 0; key_mask: device
+/* head_dim 512 (or 256); rows 16-byte aligned (ldi % 8 == 0, ldo % 4 == 0), seq_k >= 1, scale > 0; key_mask: device
  * int [seq_k] or null. `splits` and `scratch` (16-byte aligned) as the plan function of the same head_dim says for the
  * same sizes and flags; scratch may be null when it says 0 bytes. */
 extern "C" int iris_hip_fa_hd512(void *stream, uint16_t *out, int ldo, const uint16_t *q,

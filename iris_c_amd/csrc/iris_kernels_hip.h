@@ -63,16 +63,8 @@ int iris_hip_fa_hd128_qnorm(void *stream, uint16_t *out, int ldo, const uint16_t
  * the two-size grid. */
 void iris_hip_fa_hd128_plan(int seq_q, int seq_k, int heads, int causal, int *plan);
 
-/* head_dim 256 or 512 (the VAE's single 512-wide head): the head dim is cut into slices of
- * 128 that a group of waves shares; same argument conditions as iris_hip_fa_hd128. */
-int iris_hip_fa_sliced(void *stream, uint16_t *out, int ldo, const uint16_t *q,
-                       const uint16_t *k, const uint16_t *v, int ldi, int seq_q, int seq_k,
-                       int heads, int kv_heads, int head_dim, float scale, int causal,
-                       const int *key_mask);
-
-/* head_dim 512 and at least 32 keys (the VAE's call; key mask and causal limit as options): one wave per SIMD owns
- * 32 queries and all 512 output dims; the keys may be cut into ranges that a second launch merges (a causal call
- * never is). iris_hip_fa_hd512_plan says how many ranges a call of these sizes takes and returns the bytes of scratch
+/* head_dim 512 (the VAE's call; key mask and causal limit as options): one wave per SIMD owns 32 queries and all 512
+ * output dims; the keys may be cut into ranges that a second launch merges. iris_hip_fa_hd512_plan says how many ranges a call of these sizes takes and returns the bytes of scratch
  * it then needs: partial rows of the ranges, and the packed key mask of a masked call (0 for one range without mask;
  * host arithmetic, no GPU needed). iris_hip_fa_hd512 wants exactly that `splits` and a scratch of that size, 16-byte
  * aligned. Same argument conditions as iris_hip_fa_hd128 otherwise. */

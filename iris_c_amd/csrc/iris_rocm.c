@@ -306,30 +306,23 @@ void iris_dev_head_norm_rope_qk_streams(uint16_t *xq, uint16_t *xk, int ld,
                       split_half);
 }
 
-/* head_dim 256 / 512 on the matrix cores (rows 16-byte aligned). With at least 32 keys (the VAE's call at head_dim
- * 512; key mask and causal limit included) they take the kernel in which a wave owns 32 whole queries; its key
- * ranges, if it cuts any, leave their partial results in private scratch, and so does its packed key mask. Fewer
- * keys take the kernel that slices the head dim over the waves. `kind`: 0 direct, 1 through the padded copy, 2 that
- * with Q normalised. Returns 0 or a HIP error; -1 when the scratch could not be had (already reported). */
+/* head_dim 256 / 512 on the matrix cores (rows 16-byte aligned; the VAE's call at head_dim 512, key mask and causal
+ * limit included): the kernel in which a wave owns 32 whole queries. Its key ranges, if it cuts any, leave their
+ * partial results in private scratch, and so does its packed key mask. `kind`: 0 direct, 1 through the padded copy,
+ * 2 that with Q normalised. Returns 0 or a HIP error; -1 when the scratch could not be had (already reported). */
 static int attention_wide(const char *what, int kind, uint16_t *out, int ldo,
                           const uint16_t *q, const uint16_t *k, const uint16_t *v, int ldi, int seq_q, int seq_k,
                           int heads, int kv_heads, int head_dim, float scale, int causal, const int *key_mask) {
-    static const char *const names[3][3] = {{"fa_hd512", "fa_hd512_packed", "fa_hd512_packed_qnorm"},
-                                            {"fa_hd256", "fa_hd256_packed", "fa_hd256_packed_qnorm"},
-                                            {"fa_sliced", "fa_sliced_packed", "fa_sliced_packed_qnorm"}};
-    if (seq_k >= 32) {                             /* its key tiles are 32 whole rows */
-        int splits = 1;
-        const size_t need = head_dim == 512 ? iris_hip_fa_hd512_plan(seq_q, seq_k, heads, causal != 0, key_mask != NULL, &splits)
-                                            : iris_hip_fa_hd256_plan(seq_q, seq_k, heads, causal != 0, key_mask != NULL, &splits);
-        if (need && !scratch_fit(&g_split, &g_split_bytes, need, what)) return -1;
-        g_last_kernel = names[head_dim == 512 ? 0 : 1][kind];
-        return head_dim == 512
-                   ? iris_hip_fa_hd512(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal != 0, key_mask, splits, g_split)
-                   : iris_hip_fa_hd256(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal != 0, key_mask, splits, g_split);
-    }
-    g_last_kernel = names[2][kind];
-    return iris_hip_fa_sliced(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, head_dim, scale, causal != 0,
-                              key_mask);
+    static const char *const names[2][3] = {{"fa_hd512", "fa_hd512_packed", "fa_hd512_packed_qnorm"},
+                                            {"fa_hd256", "fa_hd256_packed", "fa_hd256_packed_qnorm"}};
+    int splits = 1;
+    const size_t need = head_dim == 512 ? iris_hip_fa_hd512_plan(seq_q, seq_k, heads, causal != 0, key_mask != NULL, &splits)
+                                        : iris_hip_fa_hd256_plan(seq_q, seq_k, heads, causal != 0, key_mask != NULL, &splits);
+    if (need && !scratch_fit(&g_split, &g_split_bytes, need, what)) return -1;
+    g_last_kernel = names[head_dim == 512 ? 0 : 1][kind];
+    return head_dim == 512
+               ? iris_hip_fa_hd512(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal != 0, key_mask, splits, g_split)
+               : iris_hip_fa_hd256(g_stream, out, ldo, q, k, v, ldi, seq_q, seq_k, heads, kv_heads, scale, causal != 0, key_mask, splits, g_split);
 }
 
 /* wq == NULL: plain attention. Otherwise Q is normalised and rotated on the way in. */

@@ -371,9 +371,8 @@ def test_output_stride_and_interior_pointers(dev, orc, fa):
 @pytest.mark.parametrize("seq_q,seq_k,causal,masked", [(150, 150, False, False), (1, 1, False, False), (33, 95, False, True),
                                                          (64, 64, True, False), (257, 257, True, True), (130, 1000, False, False)])
 def test_wide_heads_256_512(dev, orc, hd, heads, kv, seq_q, seq_k, causal, masked):
-    """head_dim 256 / 512 run on the matrix cores too: with at least 32 keys (the VAE's single 512-wide head; with key
-    mask and causal limit too) in the kernel whose waves own whole queries, with fewer in the kernel that slices the
-    head dim over the waves."""
+    """head_dim 256 / 512 run on the matrix cores too (the VAE's single 512-wide head; with key mask and causal limit
+    too), in the kernel whose waves own whole queries."""
     buf, ldi = random_case(hd + heads + seq_q, seq_q, seq_k, heads, kv, hd=hd)
     qd, kd = heads * hd, kv * hd
     mask = None
@@ -382,7 +381,7 @@ def test_wide_heads_256_512(dev, orc, hd, heads, kv, seq_q, seq_k, causal, maske
         mask[0] = 1                                        # every causal row keeps a valid key
     scale = float(1 / np.sqrt(hd))
     out, kernel = dev.attention(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
-    assert kernel == (f"fa_hd{hd}" if seq_k >= 32 else "fa_sliced")
+    assert kernel == f"fa_hd{hd}"
     want = orc.attention_bf16(buf, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
     assert_close(O.bf16_to_f32(out[:seq_q]), want, f"wide hd={hd} {seq_q}x{seq_k}")
 
@@ -423,13 +422,13 @@ def test_vae_shape_at_its_largest_50176_tokens(dev, orc):
     assert_close(got2[:4], np.tile(O.bf16_to_f32(buf[5, 2 * hd:]), (4, 1)), "VAE 50176 tokens constant V")
 
 
-def test_sliced_kernel_empty_rows_and_large_scores(dev, orc):
-    seq, hd = 30, 512                                   # fewer than 32 keys: the kernel that slices the head dim
+@pytest.mark.parametrize("seq,hd", [(30, 512), (100, 256), (19, 256)])
+def test_wide_heads_empty_rows_and_large_scores(dev, orc, seq, hd):
     buf, ldi = random_case(21, seq, seq, 1, 1, hd=hd, sigma=3.0)          # |score| up to ~100
     scale = float(1 / np.sqrt(hd))
     mask = np.ones(seq, np.int32); mask[:10] = 0
     out, kernel = dev.attention(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale, True, mask)
-    assert kernel == "fa_sliced"
+    assert kernel == f"fa_hd{hd}"
     got = O.bf16_to_f32(out)
     assert np.all(np.isfinite(got)) and np.all(got[:10] == 0.0)
     want = orc.attention_bf16(buf, ldi, 0, hd, 2 * hd, seq, seq, 1, 1, hd, scale, True, mask)
