@@ -422,6 +422,31 @@ def test_vae_shape_at_its_largest_50176_tokens(dev, orc):
     assert_close(got2[:4], np.tile(O.bf16_to_f32(buf[5, 2 * hd:]), (4, 1)), "VAE 50176 tokens constant V")
 
 
+@pytest.mark.parametrize("hd", [128, 256, 512, 64])
+@pytest.mark.parametrize("seq_q,seq_k", [(1, 1), (40, 5), (31, 31), (20, 33), (77, 77), (100, 1000), (700, 1027)])
+@pytest.mark.parametrize("causal,masked", [(False, False), (True, True)])
+def test_rows_behind_the_last_key_never_reach_the_output(dev, orc, hd, seq_q, seq_k, causal, masked):
+    """The kernels load K and V in tiles of 32 or 64 whole rows; what a tile holds behind the last key must not count,
+    and not by being multiplied with a zero probability either: the 48 rows that follow the last key in the buffer
+    are NaN here (q, k and v columns alike), and every output stays finite and within the bar."""
+    heads, kv = 2, 1
+    buf, ldi = random_case(hd + 3 * seq_q + seq_k, seq_q, seq_k, heads, kv, hd=hd)
+    padded = np.full((max(seq_q, seq_k) + 48, ldi), 0x7fc0, np.uint16)
+    padded[:seq_q, :heads * hd] = buf[:seq_q, :heads * hd]
+    padded[:seq_k, heads * hd:] = buf[:seq_k, heads * hd:]
+    mask = None
+    if masked:
+        mask = (np.random.default_rng(seq_k).random(seq_k) < 0.7).astype(np.int32)
+        mask[0] = 1
+    scale = float(1 / np.sqrt(hd))
+    qd, kd = heads * hd, kv * hd
+    out, _ = dev.attention(padded, ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
+    got = O.bf16_to_f32(out[:seq_q])
+    assert np.all(np.isfinite(got)), f"NaN rows {np.unique(np.argwhere(~np.isfinite(got))[:, 0])[:8]}"
+    want = orc.attention_bf16(np.ascontiguousarray(padded), ldi, 0, qd, qd + kd, seq_q, seq_k, heads, kv, hd, scale, causal, mask)
+    assert_close(got, want, f"NaN behind the keys, hd {hd} {seq_q}x{seq_k}")
+
+
 @pytest.mark.parametrize("seq,hd", [(30, 512), (100, 256), (19, 256)])
 def test_wide_heads_empty_rows_and_large_scores(dev, orc, seq, hd):
     buf, ldi = random_case(21, seq, seq, 1, 1, hd=hd, sigma=3.0)          # |score| up to ~100
