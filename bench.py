@@ -7,6 +7,7 @@ sequence: fused per-head RMSNorm + RoPE on Q, on K, then joint attention
 512 text + 4096 image token configuration, bf16, inputs resident in HBM.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle-ms T] [--no-cpu] [--no-shapes] [--no-machine]
+    python bench.py --only WIDE [--steps K]       one head of 512 / 256 dims with key masks and causal limit, 4096 - 50176 tokens
     python bench.py --only CONFIG [--steps K]     launches of one configuration only (C1 .. C5, C3-cond, C3-uncond,
                                                   VAE), for profiler runs
     python bench.py --copy-only MiB               the plain copy kernel that calibrates the byte counters
@@ -540,6 +541,38 @@ def only_one(dev, hip, stream, rng, name, steps, settle_ms):
             "flops_per_launch": fl, "tflops": round(fl / float(np.mean(ts)) / 1e9, 1)}
 
 
+def wide_heads(dev, hip, stream, rng, steps, settle_ms):
+    """One head of 512 (the VAE's call) and of 256 dims with what the device interface allows on top: a key mask that
+    leaves 60 % of the keys at random (every tile ragged), a padding mask over the last third, a causal limit, and
+    causal + mask. Average us over `steps` back-to-back calls between two events, after a settling load of the same
+    call; TFLOP/s count the (query, key) pairs the call may look at."""
+    lib, rows = dev.lib, []
+    for hd in (512, 256):
+        for seq in (4096, 16384, 50176):
+            buf = to_bf16(rng.standard_normal((seq, 3 * hd), dtype=np.float32))
+            d, o = dev.to_device(buf), lib.iris_dev_alloc(seq * hd * 2)
+            masks = {"none": None, "60 % at random": (rng.random(seq) < 0.6).astype(np.int32),
+                     "padding, last third": (np.arange(seq) < 2 * seq // 3).astype(np.int32)}
+            dm = {k: (dev.to_device(v) if v is not None else None) for k, v in masks.items()}
+            for causal, mask in ((0, "none"), (0, "60 % at random"), (0, "padding, last third"), (1, "none"), (1, "60 % at random")):
+                fn = lambda i: lib.iris_dev_attention(o, hd, d, _vp(d + 2 * hd), _vp(d + 4 * hd), 3 * hd, seq, seq, 1, 1, hd,
+                                                      float(1.0 / np.sqrt(np.float32(hd))), causal, dm[mask])
+                settle(lib, fn, settle_ms)
+                ms = event_time(hip, stream, fn, steps if seq < 50000 else max(steps // 4, 3))
+                lib.iris_dev_sync()
+                dev.check()
+                seen = (0.5 if causal else 1.0) * (2 / 3 if mask.startswith("padding") else 1.0)
+                fl = 4.0 * seq * seq * hd * seen
+                rows.append({"head_dim": hd, "tokens": seq, "causal": bool(causal), "key_mask": mask, "kernel": dev.last_kernel(),
+                             "us": round(ms * 1e3, 1), "tflops_of_visible_pairs": round(fl / ms / 1e9, 1),
+                             "frac_of_peak": round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4)})
+            for v in dm.values():
+                if v is not None:
+                    lib.iris_dev_free(v)
+            lib.iris_dev_free(d); lib.iris_dev_free(o)
+    return rows
+
+
 def occupancy_probe(dev, hip, stream, rng, settle_ms):
     """The attention kernel on one round of workgroups that fills all 256 CUs, 176 of them and 128 of them
     (4096 tokens x 16 / 11 / 8 heads: 256 / 176 / 128 workgroups of 256 queries, each walking the same 64 key
@@ -778,6 +811,9 @@ def main():
         print(json.dumps(copy_only(dev, hip, stream, args.copy_only << 20, args.steps)))
         return
 
+    if args.only == "WIDE":
+        print(json.dumps({"wide_heads": wide_heads(dev, hip, stream, rng, args.steps, min(args.settle_ms, 60))}))
+        return
     if args.only:
         print(json.dumps(only_one(dev, hip, stream, rng, args.only, args.steps, args.settle_ms)))
         return
