@@ -564,16 +564,18 @@ k_fa_fwd_hd512(uint16_t *__restrict__ out, int ldo, const uint16_t *__restrict__
 
 /* The key mask as one 32-bit word per key tile, bit j = key j of the tile AS THE KERNEL LOADS IT is valid: the last
  * tile of a sequence whose length is not a multiple of 32 is moved back to end with it, and the keys it shares with
- * the tile before count as invalid there. 64 threads = two tiles per block; `words` has room for an even count. */
-__global__ void __launch_bounds__(64)
+ * the tile before count as invalid there. 256 threads = eight tiles per block, two per wave; `words` has room for a
+ * multiple of eight. */
+__global__ void __launch_bounds__(256)
 k_pack_key_mask(uint32_t *__restrict__ words, const int *__restrict__ key_mask, int seq_k, int tiles) {
-    const int tile = 2 * blockIdx.x + (threadIdx.x >> 5), j = threadIdx.x & 31;
+    const int pair = 4 * blockIdx.x + (threadIdx.x >> 6);           /* tiles 2 pair, 2 pair + 1: one wave */
+    const int tile = 2 * pair + ((threadIdx.x >> 5) & 1), j = threadIdx.x & 31;
     const int first = max(min(tile * BN, seq_k - BN), 0), key = first + j;
     const bool ok = tile < tiles && key >= tile * BN && key < seq_k && key_mask[key] != 0;
     const unsigned long long both = __ballot(ok);
-    if (threadIdx.x == 0) {
-        words[2 * blockIdx.x] = (uint32_t)both;
-        words[2 * blockIdx.x + 1] = (uint32_t)(both >> 32);
+    if ((threadIdx.x & 63) == 0) {
+        words[2 * pair] = (uint32_t)both;
+        words[2 * pair + 1] = (uint32_t)(both >> 32);
     }
 }
 
@@ -682,7 +684,7 @@ size_t plan_ranges(int hd, int seq_q, int seq_k, int heads, int causal, int mask
     }
     *splits_out = best_s;
     const size_t rows = best_s == 1 ? 0 : (size_t)seq_q * heads * best_s;
-    const size_t words = masked ? ((size_t)tiles + 2) / 2 * 2 : 0;
+    const size_t words = masked ? ((size_t)tiles + 7) / 8 * 8 : 0;
     return rows * hd * sizeof(float) + rows * 2 * sizeof(float) + words * sizeof(uint32_t);
 }
 }  // namespace
@@ -740,7 +742,7 @@ int fa_wide(hipStream_t st, uint16_t *out, int ldo, const uint16_t *q, const uin
     uint32_t *words = nullptr;
     if (key_mask) {
         words = reinterpret_cast<uint32_t *>(reinterpret_cast<float *>(scratch) + rows * (HD + 2));
-        hipLaunchKernelGGL(k_pack_key_mask, dim3((unsigned)((tiles + 1) / 2)), dim3(64), 0, st, words, key_mask, seq_k, tiles);
+        hipLaunchKernelGGL(k_pack_key_mask, dim3((unsigned)((tiles + 7) / 8)), dim3(256), 0, st, words, key_mask, seq_k, tiles);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
     }

@@ -247,7 +247,7 @@ def launch_with_ranges(dev, buf, ldi, seq_q, seq_k, heads, kv, scale, splits, ca
     d = dev.put(buf)
     out0 = np.full((seq_q, qd), 0x7fc0, dtype=np.uint16)
     do = dev.put(out0)
-    scratch = dev.alloc(max(16, seq_q * heads * splits * (hd + 2) * 4) + 4 * ((seq_k + 31) // 32 + 2))
+    scratch = dev.alloc(max(16, seq_q * heads * splits * (hd + 2) * 4) + 4 * ((seq_k + 31) // 32 + 8))
     dm = dev.put(np.ascontiguousarray(mask, np.int32)) if mask is not None else None
     err = run(lib.iris_dev_stream(), do, qd, d, ptr_add(d, 2 * qd), ptr_add(d, 2 * (qd + kd)), ldi, seq_q, seq_k,
                                 heads, kv, scale, int(causal), dm, splits, scratch)
@@ -347,7 +347,7 @@ def test_planner_never_leaves_a_range_empty():
                 tiles = (seq_k + 31) // 32
                 per = (tiles + splits - 1) // splits
                 assert 1 <= splits <= min(8, tiles) and (tiles + per - 1) // per == splits, (seq_q, seq_k, heads, splits)
-                words = (tiles + 2) // 2 * 2 if masked else 0       # one word per tile, an even count, one pair to spare
+                words = (tiles + 7) // 8 * 8 if masked else 0       # one word per tile, a multiple of eight
                 assert need == (0 if splits == 1 else seq_q * heads * splits * (HD + 2) * 4) + 4 * words
     assert plan(lib, 16384, 16384, 1)[0] == 2                 # 128 workgroups of 128 queries on 256 CUs
     assert plan(lib, 128, 64, 1)[0] == 1
